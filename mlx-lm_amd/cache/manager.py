@@ -16,7 +16,7 @@ cut into pages of ``page_size`` tokens instead:
 * Pages are taken before a step runs (``reserve``) and counted as filled after
   it (``commit``); they are given back when the request ends (``release``), is
   cut short (``truncate``) or, in a windowed group, when every later query is
-  out of their reach.
+  out of their reach (the pages of the first ``keep_first`` tokens never are).
 * Every request also gets a state slot: a row in each fixed-size state tensor
   (zeroed when the request starts), whether or not any mixer asks for one.
 * What a request computed can be kept beyond its end (``detach``) for a later
@@ -225,9 +225,10 @@ class CacheManager:
             w = g.need.window
             if w <= 0:
                 continue
-            # the next query sits at position >= length and sees keys > position - w
+            # the next query sits at position >= length and sees keys > position - w,
+            # and the first keep_first keys whatever its position
             first_needed = max(0, rc.length - w + 1)
-            for b in range(first_needed // self.page_size):
+            for b in range(self.blocks_for(g.need.keep_first), first_needed // self.page_size):
                 if rc.blocks[gi][b] >= 0:
                     g.pool.give_back([rc.blocks[gi][b]])
                     rc.blocks[gi][b] = -1
@@ -249,7 +250,7 @@ class CacheManager:
             w = g.need.window
             if w > 0:
                 first_needed = max(0, new_length - w + 1) // self.page_size
-                if any(p < 0 for p in rc.blocks[gi][first_needed:keep]):
+                if any(p < 0 for p in rc.blocks[gi][first_needed:keep]):  # (the kept first pages never went)
                     raise ValueError(
                         f"request {request_id!r}: a window has already dropped pages that "
                         f"length {new_length} needs"

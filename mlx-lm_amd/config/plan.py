@@ -24,10 +24,13 @@ class PartSpec:
 class LayerSpec:
     """One layer: an arrangement (block kind) and the parts it arranges, by the names
     that the arrangement gives them (``pre_norm``: ``mixer_norm``, ``mixer``, ``ffn_norm``,
-    ``ffn``).  Which parts there are, and how many, is the arrangement's business."""
+    ``ffn``).  Which parts there are, and how many, is the arrangement's business; ``params`` are
+    the arrangement's own constants and options (``post_norm``: ``alpha``, ``layer_scale``,
+    ``token_shift``, the prefix of its tensors)."""
 
     arrangement: str
     parts: Dict[str, PartSpec]
+    params: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -38,11 +41,14 @@ class RunEntry:
     schedule.  ``cache`` names the cache slot that this run's mixer reads; two
     runs that name the same slot share keys and values, and only the run with
     ``writes_cache`` puts this step's tokens there (it has to come first).
+    ``state`` names a second slot, of per-request state that the layer's
+    arrangement itself keeps for this run (``Block.state_need()``), or ``None``.
     """
 
     layer: int
     cache: int
     writes_cache: bool = True
+    state: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -53,6 +59,7 @@ class CacheNeed:
     head_dim: int  # width of a head's key
     window: int = 0  # 0: every earlier token; n: the last n tokens
     v_head_dim: int = 0  # width of a head's value; 0: as the key's
+    keep_first: int = 0  # with a window: the first so many tokens stay visible (and keep their pages)
 
     @property
     def value_dim(self):
@@ -93,11 +100,14 @@ class ModelPlan:
                 raise ValueError(
                     f"schedule entry {i} reads cache slot {run.cache} before any run has written it"
                 )
-        slots = sorted(written)
+        states = [run.state for run in self.schedule if run.state is not None]
+        if len(set(states)) != len(states) or set(states) & written:
+            raise ValueError("a run's state slot is its own: no other run's state, no run's cache")
+        slots = sorted(written | set(states))
         if slots != list(range(len(slots))):
             raise ValueError(f"cache slots must be numbered 0..n-1 without gaps, got {slots}")
         return self
 
     @property
     def n_cache_slots(self):
-        return len({run.cache for run in self.schedule})
+        return len({run.cache for run in self.schedule} | {run.state for run in self.schedule if run.state is not None})

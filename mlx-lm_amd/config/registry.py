@@ -6,7 +6,7 @@ import importlib
 MODEL_REMAPPING = {}
 
 _REGISTRY = {}
-_BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2"}
+_BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2", "pafutar": "mlx_lm_amd.models.pafutar"}
 
 
 def register_model(model_type, model_cls, args_cls):
@@ -18,13 +18,22 @@ def registered_model_types():
     return sorted(set(_REGISTRY) | set(_BUILTIN))
 
 
+def model_type_of(config):
+    """The registry key of a configuration: its ``model_type``, or, where a config.json names
+    its design under ``architecture`` instead, that name in lower case."""
+    model_type = config.get("model_type")
+    if model_type is None and isinstance(config.get("architecture"), str):
+        model_type = config["architecture"].lower()
+    return model_type
+
+
 def get_model_classes(config):
     """``(Model, ModelArgs)`` for ``config["model_type"]``.
 
     Follows mlx_lm/utils.py:177-195: aliases first, then the architecture's
     module; an unknown type is a ``ValueError`` with the reference's text.
     """
-    model_type = config.get("model_type")
+    model_type = model_type_of(config)
     model_type = MODEL_REMAPPING.get(model_type, model_type)
     if model_type in _REGISTRY:
         return _REGISTRY[model_type]

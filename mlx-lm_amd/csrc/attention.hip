@@ -43,7 +43,39 @@ struct AttnArgs {
   int window;
   int n_splits;
   float scale;
+  // Optional terms of a score and of the output (all absent: plain causal attention).
+  //   head_scale [n_heads]: head h's scores are q.k * head_scale[h] instead of q.k * scale
+  //   slopes [n_heads]: slope[h] * (query position - key position) is taken off the score
+  //   keep_first: with a window, keys at positions below it stay visible to every later query
+  //   gate [n_tokens, n_heads*head_dim] (row stride ldg): the output is multiplied by sigmoid(gate)
+  const float* head_scale;
+  const float* slopes;
+  const void* gate;
+  int ldg, keep_first;
 };
+
+// The two runs of keys that the queries at positions q_lo .. (whose last key is k_hi - 1) read:
+// the kept first keys [0, sink_hi) and the window's [k_lo, k_hi).  Without a window: one run.
+struct KeyRuns {
+  int sink_hi, k_lo, k_hi;
+};
+__device__ __forceinline__ KeyRuns key_runs(const AttnArgs& p, int q_lo, int k_hi) {
+  KeyRuns r;
+  r.k_hi = k_hi;
+  r.k_lo = p.window > 0 ? max(0, q_lo - p.window + 1) : 0;
+  r.sink_hi = min(p.keep_first, r.k_lo);
+  return r;
+}
+// Whether the query at qpos sees the key at kpos (kpos <= qpos is checked by the caller's k_hi too).
+__device__ __forceinline__ bool sees(const AttnArgs& p, int qpos, int kpos) {
+  return kpos <= qpos && (p.window <= 0 || qpos - kpos < p.window || kpos < p.keep_first);
+}
+__device__ __forceinline__ float gate_of(const AttnArgs& p, int row, int col, bool is_bf16) {
+  if (!p.gate) return 1.f;
+  const size_t i = (size_t)row * p.ldg + col;
+  const float g = is_bf16 ? bits_to_f32(((const uint16_t*)p.gate)[i]) : ((const float*)p.gate)[i];
+  return 1.0f / (1.0f + expf(-g));
+}
 
 #define KT 64   // keys per tile
 #define QT ATTN_TILE_QUERIES  // queries per block in attn_tile
@@ -180,15 +212,18 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
   const T* q = (const T*)p.q;
   const T* k_pages = (const T*)p.k_pages;
   const T* v_pages = (const T*)p.v_pages;
+  const float q_scale = p.head_scale ? p.head_scale[h] : p.scale;
+  const float slope = p.slopes ? p.slopes[h] : 0.f;
 
   for (int c = tid; c < QT * hd; c += 256) {
     const int qi = c / hd, d = c - qi * hd;
-    Qs[c] = qi < nq ? to_f32(q[(size_t)(row0 + qi) * p.ldq + h * hd + d]) * p.scale : 0.f;
+    Qs[c] = qi < nq ? to_f32(q[(size_t)(row0 + qi) * p.ldq + h * hd + d]) * q_scale : 0.f;
   }
 
-  const int k_hi = pos0 + nq;  // one past the last key any query of the tile sees
-  const int k_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
-  const int kt0 = (k_lo / KT) * KT;
+  const KeyRuns runs = key_runs(p, pos0, pos0 + nq);  // (k_hi: one past the last key any query of the tile sees)
+  const int n_sink_tiles = (runs.sink_hi + KT - 1) / KT;
+  const int kt0 = (runs.k_lo / KT) * KT;
+  const int n_tiles_all = n_sink_tiles + (runs.k_hi - kt0 + KT - 1) / KT;
 
   float m[4], l[4], o[4][4];
 #pragma unroll
@@ -198,7 +233,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
     for (int j = 0; j < 4; ++j) o[i][j] = 0.f;
   }
 
-  for (int kt = kt0; kt < k_hi; kt += KT) {
+  for (int t = 0; t < n_tiles_all; ++t) {
+    // the kept first keys' tiles, then the window's
+    const bool sink = t < n_sink_tiles;
+    const int kt = sink ? t * KT : kt0 + (t - n_sink_tiles) * KT;
+    const int k_lo = sink ? 0 : runs.k_lo, k_hi = sink ? runs.sink_hi : runs.k_hi;
     __syncthreads();  // previous tile's values are no longer read; Qs is written
     stage_tile<T>(KVs, kv_stride, k_pages, table, p, kv_head, kt, k_lo, k_hi, tid, 256);
     __syncthreads();
@@ -214,9 +253,8 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
         const float4 qv = *(const float4*)(qrow + d);
         s += qv.x * krow[d] + qv.y * krow[d + 1] + qv.z * krow[d + 2] + qv.w * krow[d + 3];
       }
-      bool ok = qi < nq && kpos <= qpos && kpos >= k_lo;
-      if (p.window > 0) ok = ok && kpos > qpos - p.window;
-      s = ok ? s : -INFINITY;
+      const bool ok = qi < nq && kpos >= k_lo && kpos < k_hi && sees(p, qpos, kpos);
+      s = ok ? s - slope * (float)(qpos - kpos) : -INFINITY;
       const float m_new = fmaxf(m[i], wave_max(s));
       float pr = 0.f, alpha = 1.f;
       if (m_new != -INFINITY) {
@@ -256,7 +294,9 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int d = lane + 64 * j;
-      if (d < hd) out[(size_t)(row0 + qi) * p.ldo + h * hd + d] = from_f32<T>(o[i][j] * inv);
+      if (d < hd)
+        out[(size_t)(row0 + qi) * p.ldo + h * hd + d] =
+            from_f32<T>(o[i][j] * inv * gate_of(p, row0 + qi, h * hd + d, sizeof(T) == 2));
     }
   }
 }
@@ -437,12 +477,14 @@ __global__ __launch_bounds__(256) void attn_row_kernel(AttnArgs p) {
   const T* k_pages = (const T*)p.k_pages;
   const T* v_pages = (const T*)p.v_pages;
 
-  for (int d = tid; d < hd; d += 256) Qs[d] = to_f32(q[(size_t)row * p.ldq + h * hd + d]) * p.scale;
+  const float q_scale = p.head_scale ? p.head_scale[h] : p.scale;
+  const float slope = p.slopes ? p.slopes[h] : 0.f;
+  for (int d = tid; d < hd; d += 256) Qs[d] = to_f32(q[(size_t)row * p.ldq + h * hd + d]) * q_scale;
 
-  const int k_hi = pos + 1;
-  const int k_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
-  const int kt0 = (k_lo / KT) * KT;
-  const int n_tiles = (k_hi - kt0 + KT - 1) / KT;
+  const KeyRuns runs = key_runs(p, pos, pos + 1);
+  const int n_sink_tiles = (runs.sink_hi + KT - 1) / KT;  // the kept first keys' tiles come first
+  const int kt0 = (runs.k_lo / KT) * KT;
+  const int n_tiles = n_sink_tiles + (runs.k_hi - kt0 + KT - 1) / KT;
   const int tiles_per_split = (n_tiles + p.n_splits - 1) / p.n_splits;
   const int t_begin = split * tiles_per_split;
   const int t_end = min(n_tiles, t_begin + tiles_per_split);
@@ -454,7 +496,9 @@ __global__ __launch_bounds__(256) void attn_row_kernel(AttnArgs p) {
   for (int r = 0; r < rounds; ++r) {
     const int tile = t_begin + r * 4 + wave;
     const bool active = tile < t_end;
-    const int kt = kt0 + tile * KT;
+    const bool sink = tile < n_sink_tiles;
+    const int kt = sink ? tile * KT : kt0 + (tile - n_sink_tiles) * KT;
+    const int k_lo = sink ? 0 : runs.k_lo, k_hi = sink ? runs.sink_hi : runs.k_hi;
     if (active) stage_tile<T>(KVs, kv_stride, k_pages, table, p, kv_head, kt, k_lo, k_hi, lane, 64);
     __syncthreads();
     if (active) {
@@ -466,7 +510,7 @@ __global__ __launch_bounds__(256) void attn_row_kernel(AttnArgs p) {
         s += qv.x * krow[d] + qv.y * krow[d + 1] + qv.z * krow[d + 2] + qv.w * krow[d + 3];
       }
       const bool ok = kpos >= k_lo && kpos < k_hi;
-      s = ok ? s : -INFINITY;
+      s = ok ? s - slope * (float)(pos - kpos) : -INFINITY;
       const float m_new = fmaxf(m, wave_max(s));
       float pr = 0.f, alpha = 1.f;
       if (m_new != -INFINITY) {
@@ -516,7 +560,8 @@ __global__ __launch_bounds__(256) void attn_row_kernel(AttnArgs p) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc += Os[i * hd + d] * w[i];
     if (p.n_splits == 1) {
-      ((T*)p.out)[(size_t)row * p.ldo + h * hd + d] = from_f32<T>(acc / L);
+      ((T*)p.out)[(size_t)row * p.ldo + h * hd + d] =
+          from_f32<T>(acc / L * gate_of(p, row, h * hd + d, sizeof(T) == 2));
     } else {
       const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
       p.part_o[base * hd + d] = acc;
@@ -545,7 +590,8 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(AttnArgs p) {
       const float ms = p.part_ml[(base + s) * 2];
       if (ms != -INFINITY) acc += p.part_o[(base + s) * hd + d] * expf(ms - M);
     }
-    ((T*)p.out)[(size_t)row * p.ldo + h * hd + d] = from_f32<T>(acc / L);
+    ((T*)p.out)[(size_t)row * p.ldo + h * hd + d] =
+        from_f32<T>(acc / L * gate_of(p, row, h * hd + d, sizeof(T) == 2));
   }
 }
 
@@ -558,8 +604,8 @@ static int check_geometry(const char* who, int n_heads, int n_kv_heads, int head
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("%s: unknown dtype code %d", who, dtype);
   if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
     FAIL("%s: %d query heads cannot be grouped over %d key heads", who, n_heads, n_kv_heads);
-  if (head_dim < 16 || head_dim > 256 || head_dim % 16 != 0)
-    FAIL("%s: head_dim %d must be a multiple of 16 between 16 and 256", who, head_dim);
+  if (head_dim < 8 || head_dim > 256 || head_dim % 8 != 0)
+    FAIL("%s: head_dim %d must be a multiple of 8 between 8 and 256", who, head_dim);
   if (page_size <= 0) FAIL("%s: page_size %d must be positive", who, page_size);
   return 0;
 }
@@ -623,8 +669,20 @@ static int fill_args(AttnArgs& p, const char* who, void* out, const void* q, int
   p.page_stride = page_stride, p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.head_dim = head_dim, p.page_size = page_size;
   p.window = window, p.n_splits = 1, p.scale = scale;
+  p.head_scale = nullptr, p.slopes = nullptr, p.gate = nullptr, p.ldg = 0, p.keep_first = 0;
   return 0;
 }
+
+// The optional terms (AttnArgs): any of the pointers may be null.
+static int fill_extras(AttnArgs& p, const char* who, const float* head_scale, const float* slopes,
+                       const void* gate, int ldg, int keep_first) {
+  if (keep_first < 0) FAIL("%s: keep_first %d must not be negative", who, keep_first);
+  if (gate && ldg < p.n_heads * p.head_dim) FAIL("%s: the gate's row stride %d is smaller than its rows", who, ldg);
+  p.head_scale = head_scale, p.slopes = slopes, p.gate = gate, p.ldg = ldg;
+  p.keep_first = p.window > 0 ? keep_first : 0;  // (without a window every key is visible anyway)
+  return 0;
+}
+static bool has_extras(const AttnArgs& p) { return p.head_scale || p.slopes || p.gate || p.keep_first > 0; }
 
 // Kernels that want more than 64 KB of LDS have to be told so once per size.
 static int allow_lds(const char* who, const void* kernel, size_t bytes) {
@@ -645,18 +703,23 @@ static int allow_lds(const char* who, const void* kernel, size_t bytes) {
 
 // items: n_tiles pairs (first flat row, number of rows 1..16); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
-extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                         const void* v_pages, size_t page_stride, const int* block_table,
-                         int max_blocks, const int* token_req, const int* positions,
-                         const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
-                         int page_size, int window, float scale, int dtype, hipStream_t stream) {
+// attn_tile_biased: attn_tile with the optional terms of AttnArgs (per-head scales, distance
+// slopes, kept first keys, an output gate; null or 0 where a term is absent).
+extern "C" int attn_tile_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                const void* v_pages, size_t page_stride, const int* block_table,
+                                int max_blocks, const int* token_req, const int* positions,
+                                const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
+                                int page_size, int window, float scale, int dtype, const float* head_scale,
+                                const float* slopes, const void* gate, int ldg, int keep_first,
+                                hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   AttnArgs p;
   if (fill_args(p, "attn_tile", out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table,
                 max_blocks, token_req, positions, tiles, n_heads, n_kv_heads, head_dim, page_size,
                 window, scale, dtype))
     return 1;
-  if (dtype == DT_F32 && (head_dim == 64 || head_dim == 128) && page_size % 16 == 0 && ldq % 4 == 0 &&
+  if (fill_extras(p, "attn_tile", head_scale, slopes, gate, ldg, keep_first)) return 1;
+  if (!has_extras(p) && dtype == DT_F32 && (head_dim == 64 || head_dim == 128) && page_size % 16 == 0 && ldq % 4 == 0 &&
       ldo % 4 == 0 && (((uintptr_t)q | (uintptr_t)out) & 15) == 0) {
     dim3 grid((n_tiles + 3) / 4, n_heads), block(256);
     if (head_dim == 64)
@@ -679,21 +742,33 @@ extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void*
   return 0;
 }
 
+extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                         const void* v_pages, size_t page_stride, const int* block_table,
+                         int max_blocks, const int* token_req, const int* positions,
+                         const int* tiles, int n_tiles, int n_heads, int n_kv_heads, int head_dim,
+                         int page_size, int window, float scale, int dtype, hipStream_t stream) {
+  return attn_tile_biased(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                          positions, tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                          dtype, nullptr, nullptr, nullptr, 0, 0, stream);
+}
+
 // rows: n_rows flat row indices, each handled as a single query.  With
 // n_splits > 1 the caller gives part_o [n_rows*n_heads*n_splits*head_dim] and
 // part_ml [n_rows*n_heads*n_splits*2] floats.
-extern "C" int attn_row(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                        const void* v_pages, size_t page_stride, const int* block_table,
-                        int max_blocks, const int* token_req, const int* positions,
-                        const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                        int page_size, int window, float scale, int n_splits, float* part_o,
-                        float* part_ml, int dtype, hipStream_t stream) {
+extern "C" int attn_row_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                               const void* v_pages, size_t page_stride, const int* block_table,
+                               int max_blocks, const int* token_req, const int* positions,
+                               const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                               int page_size, int window, float scale, int n_splits, float* part_o,
+                               float* part_ml, int dtype, const float* head_scale, const float* slopes,
+                               const void* gate, int ldg, int keep_first, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   AttnArgs p;
   if (fill_args(p, "attn_row", out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table,
                 max_blocks, token_req, positions, rows, n_heads, n_kv_heads, head_dim, page_size,
                 window, scale, dtype))
     return 1;
+  if (fill_extras(p, "attn_row", head_scale, slopes, gate, ldg, keep_first)) return 1;
   if (n_splits < 1 || n_splits > 65535) FAIL("attn_row: n_splits %d out of range", n_splits);
   if (n_splits > 1 && (!part_o || !part_ml)) FAIL("attn_row: splits need the partial buffers");
   p.n_splits = n_splits, p.part_o = part_o, p.part_ml = part_ml;
@@ -713,4 +788,15 @@ extern "C" int attn_row(void* out, const void* q, int ldq, int ldo, const void* 
   }
   CHECK_LAUNCH("attn_row");
   return 0;
+}
+
+extern "C" int attn_row(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                        const void* v_pages, size_t page_stride, const int* block_table,
+                        int max_blocks, const int* token_req, const int* positions,
+                        const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                        int page_size, int window, float scale, int n_splits, float* part_o,
+                        float* part_ml, int dtype, hipStream_t stream) {
+  return attn_row_biased(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                         positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                         n_splits, part_o, part_ml, dtype, nullptr, nullptr, nullptr, 0, 0, stream);
 }

@@ -116,6 +116,23 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// The activations that a product's epilogue can apply, chosen by two of its flag bits
+// (the same bits in every product kernel): tanh-GELU, or the square of the ReLU.
+#define FLAG_ACT_GELU 1
+#define FLAG_ACT_RELU2 32
+#define FLAG_ACT_ANY (FLAG_ACT_GELU | FLAG_ACT_RELU2)
+__device__ __forceinline__ float relu_squared(float x) {
+  const float r = fmaxf(x, 0.f);
+  return r * r;
+}
+// `fast`: the GELU on the hardware's exponential, for results that are rounded to bfloat16 anyway
+template <bool FAST>
+__device__ __forceinline__ float activate(int flags, float v) {
+  if (flags & FLAG_ACT_GELU) return FAST ? gelu_tanh_fast(v) : gelu_tanh(v);
+  if (flags & FLAG_ACT_RELU2) return relu_squared(v);
+  return v;
+}
+
 // Sum over a block of up to 1024 threads; `red` is LDS of at least 17 floats.
 // Every thread gets the result.  Safe to call repeatedly with the same `red`.
 __device__ __forceinline__ float block_sum(float v, float* red) {

@@ -162,17 +162,18 @@ EngPart* eng_make_attention(int width, int n_heads, int n_kv_heads, int head_dim
 EngPart* eng_make_gelu_mlp(int width, int inner_padded, const EngWeight* fc_w, const float* fc_b,
                            const EngWeight* proj_w, const float* proj_b);
 EngPart* eng_make_pre_norm_block(EngPart* mixer_norm, EngPart* mixer, EngPart* ffn_norm, EngPart* ffn);
-EngPart* eng_make_token_embedding(const void* table, int vocab, int width, int dtype);
+EngPart* eng_make_token_embedding(const void* table, int vocab, int width, int dtype, float scale);
 EngPart* eng_make_learned_positions(const void* table, int max_positions, int width, int dtype);
 EngPart* eng_make_linear_head(const EngWeight* w);
 EngPart* eng_make_model(int width, int vocab, EngPart* embedding, EngPart* positions, int n_layers,
                         EngPart** layers, int n_runs, const int* run_layer, const int* run_cache,
-                        const int* run_writes, EngPart* final_norm, EngPart* head);
+                        const int* run_writes, const int* run_state, EngPart* final_norm, EngPart* head);
 void eng_free(EngPart* part);
 
 // Each returns 0, or 1 with the text in mlxlm_last_error() (2: a callback kept a Python exception).
 int eng_model_forward(EngPart* model, EngCtx* ctx);
-int eng_block_forward(EngPart* block, EngCtx* ctx, const EngMat* h, int cache_slot, int writes_cache);
+int eng_block_forward(EngPart* block, EngCtx* ctx, const EngMat* h, int cache_slot, int writes_cache,
+                      int state_slot);
 int eng_norm_forward(EngPart* norm, EngCtx* ctx, const EngMat* x, const int* rows, int n_rows, int lazy,
                      const EngWeight* ahead, EngValue* out);
 int eng_mixer_forward(EngPart* mixer, EngCtx* ctx, const EngValue* x, const EngMat* residual, int cache_slot,
@@ -200,7 +201,7 @@ typedef struct {
   EngWeight w;
   const float* bias;
   const EngScatter* scatter;
-  int gelu, accumulate, variant, splits;  // splits: 0 = the library chooses
+  int gelu, accumulate, variant, splits;  // gelu: the activation (0 none, 1 tanh-GELU, 2 squared ReLU); splits: 0 = the library chooses
   int out_packed, pad_;  // out (bfloat16, [rows padded to 16][cols padded to 64]) in the packed order
 } EngLinear;
 int eng_linear(EngCtx* ctx, const EngLinear* call, EngPending* pending);

@@ -29,6 +29,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 #define DECODE_MAX_ROWS 16
 #define F32_FEW_ROWS 64  // rows that the 32-bit product's streaming kernel takes
 #define GEMM_OUT_PACKED 16
+#define GEMM_RELU2 32  // the square of the ReLU (an activation code of 2)
 #define ROWS_MAX_ROWS 64  // up to here the kernel for 17 to 64 rows
 #define ATTN_ROW_MAX_HEAD_DIM 144
 #define READ_AHEAD_BYTES_PER_CU (160 * 1024)  // what an idle CU reads while decode attention runs
@@ -75,7 +76,7 @@ struct Entry {
   }
 };
 
-typedef int (*fn_embed)(void*, const void*, const int*, const void*, const int*, int, int, int, hipStream_t);
+typedef int (*fn_embed)(void*, const void*, const int*, const void*, const int*, int, int, int, float, hipStream_t);
 typedef int (*fn_layernorm)(void*, const float*, const int*, const float*, const float*, float, int, int, int,
                             hipStream_t);
 typedef int (*fn_gemm_f32)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
@@ -114,7 +115,7 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
 
-static Entry<fn_embed> k_embed("embed", "embed_gather_add");
+static Entry<fn_embed> k_embed("embed", "embed_scale_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
 static Entry<fn_gemm_f32> k_gemm_f32("gemm_f32", "gemm_f32");
 static Entry<fn_int4> k_gemm_f32_splits("gemm_f32", "gemm_f32_splits");
@@ -196,9 +197,12 @@ static inline bool waits_on(const EngPending& p, const EngMat& x) {
   return p.target != nullptr && (void*)p.target == x.p && p.rows == x.rows && p.cols == x.cols;
 }
 
+// An activation code (0 none, 1 tanh-GELU, 2 squared ReLU) as the product kernels' flag bits.
+static inline int act_flags(int act) { return act == 1 ? GEMM_GELU : act == 2 ? GEMM_RELU2 : 0; }
+
 static int sum_partials(EngCtx* ctx, const EngMat& out, const float* ws, int n_splits, const float* bias,
-                        bool gelu, bool accumulate, const EngScatter* sc, bool out_packed = false) {
-  int flags = (gelu ? GEMM_GELU : 0) | (accumulate ? GEMM_ACCUMULATE : 0) | (out_packed ? GEMM_OUT_PACKED : 0);
+                        int act, bool accumulate, const EngScatter* sc, bool out_packed = false) {
+  int flags = act_flags(act) | (accumulate ? GEMM_ACCUMULATE : 0) | (out_packed ? GEMM_OUT_PACKED : 0);
   if (out.dtype == DT_F32) {
     if (!accumulate) flags |= GEMM_OUT_F32;
   } else if (accumulate) {
@@ -218,7 +222,7 @@ static int settle(EngCtx* ctx, EngPending* p) {
   EngMat target = {p->target, p->rows, p->cols, p->ld, DT_F32};
   p->target = nullptr;
   if (ctx->stats) ctx->stats->settle_plain++;
-  return sum_partials(ctx, target, p->ws, p->n_splits, p->bias, false, true, nullptr);
+  return sum_partials(ctx, target, p->ws, p->n_splits, p->bias, 0, true, nullptr);
 }
 
 extern "C" int eng_settle(EngCtx* ctx) { return settle(ctx, &ctx->pending); }
@@ -318,7 +322,7 @@ extern "C" int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, i
 // What follows a product that left K in parts in the workspace: the sum stays pending where it
 // goes into the residual stream and the caller allows that (the next norm adds it), otherwise
 // the second kernel adds the parts and runs the epilogue.
-static int finish_parts(EngCtx* ctx, const EngMat& out, float* ws, int n_splits, const float* bias, bool gelu,
+static int finish_parts(EngCtx* ctx, const EngMat& out, float* ws, int n_splits, const float* bias, int gelu,
                         bool accumulate, const EngScatter* sc, EngPending* pending, bool out_packed = false) {
   if (accumulate && pending && pending->allowed) {
     pending->target = (float*)out.p, pending->rows = out.rows, pending->cols = out.cols, pending->ld = out.ld;
@@ -365,8 +369,9 @@ extern "C" int eng_wants_packed_rows(const EngCtx* ctx, const EngWeight* w, int 
   return wants_packed(ctx, n_rows, w) ? 1 : 0;
 }
 
+// `gelu`: the activation code of the epilogue (0 none, 1 tanh-GELU, 2 squared ReLU).
 static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWeight& w, const float* bias,
-                  bool gelu, bool accumulate, int variant, const EngScatter* sc, int splits,
+                  int gelu, bool accumulate, int variant, const EngScatter* sc, int splits,
                   EngPending* pending, bool out_packed = false) {
   const int M = a.m.rows, K = a.m.cols, N = w.N;
   if (a.packed && a.lazy) FAIL("linear: a norm not computed yet has no packed rows");
@@ -377,7 +382,8 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
     FAIL("linear: a and w must share float32 or bfloat16");
   if (!w.w && !(w.packed && w.dtype == DT_BF16)) FAIL("linear: the weights have no memory");
   if (M == 0) return 0;
-  int flags = gelu ? GEMM_GELU : 0;
+  if (gelu < 0 || gelu > 2) FAIL("linear: unknown activation code %d", gelu);
+  int flags = act_flags(gelu);
   if (accumulate) {
     if (out.dtype != DT_F32) FAIL("linear: accumulate needs a float32 out");
     flags |= GEMM_ACCUMULATE;
@@ -516,7 +522,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
 }
 
 extern "C" int eng_linear(EngCtx* ctx, const EngLinear* c, EngPending* pending) {
-  return linear(ctx, c->out, c->a, c->w, c->bias, c->gelu != 0, c->accumulate != 0, c->variant, c->scatter,
+  return linear(ctx, c->out, c->a, c->w, c->bias, c->gelu, c->accumulate != 0, c->variant, c->scatter,
                 c->splits, pending, c->out_packed != 0);
 }
 
@@ -591,7 +597,7 @@ struct PyFeedForward : FeedForward {
 struct PyBlock : Block {
   int id;
   PyBlock(int i, int flags) : id(i) { handles_pending = false, (void)flags; }
-  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes) override {
+  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int) override {
     EngCall c = {};
     c.residual = h, c.cache_slot = slot, c.writes_cache = writes;
     return call_python(id, ENG_CB_BLOCK, ctx, &c);
@@ -905,7 +911,7 @@ struct PreNormBlock : Block {
     return norm->forward(ctx, h, nullptr, 0, lazy, norm->reads_ahead ? first : nullptr, may_pack, x);
   }
 
-  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes) override {
+  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int) override {
     const size_t mark = ctx->scratch->offset;
     EngValue x;
     TRY(normed(ctx, mixer_norm, h, mixer->accepts_lazy, mixer->accepts_packed, mixer->first_weight, &x));
@@ -926,12 +932,13 @@ struct PreNormBlock : Block {
 struct TokenEmbedding : Embedding {
   const void* table;
   int vocab, width, dtype;
+  float scale;  // the token's row is multiplied by it (the added row is not)
   int forward(EngCtx* ctx, const EngMat& out, const EngMat& add_table, const int* add_index) override {
     if (out.cols != width || out.dtype != DT_F32 || out.ld != width) FAIL("embedding: out must be float32 [tokens, %d]", width);
     if (add_table.p && (add_table.cols != width || add_table.dtype != dtype))
       FAIL("embedding: the position table must share the token table's width and dtype");
     KERNEL(k_embed, ctx, out.p, table, ctx->token_ids, add_table.p, add_table.p ? add_index : nullptr, out.rows,
-           width, dtype, ctx->stream);
+           width, dtype, scale, ctx->stream);
     return 0;
   }
 };
@@ -956,7 +963,7 @@ struct LinearHead : Head {
 // -- the model ---------------------------------------------------------------------
 
 struct Run {
-  int layer, cache, writes;
+  int layer, cache, writes, state;
 };
 
 struct Model : EngPart {
@@ -983,7 +990,7 @@ struct Model : EngPart {
       // a block that does not know of pending sums gets the stream with everything added
       pending->allowed = block->handles_pending;
       if (!pending->allowed) TRY(settle(ctx, pending));
-      TRY(block->forward(ctx, h, run.cache, run.writes != 0));
+      TRY(block->forward(ctx, h, run.cache, run.writes != 0, run.state));
     }
     pending->allowed = 0;
     if (ctx->n_wanted == 0 || !final_norm->settles_pending) TRY(settle(ctx, pending));
@@ -1119,9 +1126,9 @@ extern "C" EngPart* eng_make_pre_norm_block(EngPart* mixer_norm, EngPart* mixer,
   return b;
 }
 
-extern "C" EngPart* eng_make_token_embedding(const void* table, int vocab, int width, int dtype) {
+extern "C" EngPart* eng_make_token_embedding(const void* table, int vocab, int width, int dtype, float scale) {
   TokenEmbedding* e = new TokenEmbedding();
-  e->table = table, e->vocab = vocab, e->width = width, e->dtype = dtype;
+  e->table = table, e->vocab = vocab, e->width = width, e->dtype = dtype, e->scale = scale;
   return e;
 }
 
@@ -1139,7 +1146,8 @@ extern "C" EngPart* eng_make_linear_head(const EngWeight* w) {
 
 extern "C" EngPart* eng_make_model(int width, int vocab, EngPart* embedding, EngPart* positions, int n_layers,
                                    EngPart** layers, int n_runs, const int* run_layer, const int* run_cache,
-                                   const int* run_writes, EngPart* final_norm, EngPart* head) {
+                                   const int* run_writes, const int* run_state, EngPart* final_norm,
+                                   EngPart* head) {
   std::unique_ptr<Model> m(new Model());
   m->width = width, m->vocab = vocab;
   if (!(m->embedding = as<Embedding>(embedding, KIND_EMBEDDING, "eng_make_model"))) return nullptr;
@@ -1155,7 +1163,7 @@ extern "C" EngPart* eng_make_model(int width, int vocab, EngPart* embedding, Eng
       snprintf(g_err, sizeof(g_err), "eng_make_model: run %d names layer %d of %d", i, run_layer[i], n_layers);
       return nullptr;
     }
-    m->schedule.push_back(Run{run_layer[i], run_cache[i], run_writes[i]});
+    m->schedule.push_back(Run{run_layer[i], run_cache[i], run_writes[i], run_state ? run_state[i] : -1});
   }
   if (!(m->final_norm = as<Norm>(final_norm, KIND_NORM, "eng_make_model"))) return nullptr;
   if (!(m->head = as<Head>(head, KIND_HEAD, "eng_make_model"))) return nullptr;
@@ -1170,9 +1178,9 @@ extern "C" int eng_model_forward(EngPart* model, EngCtx* ctx) {
 }
 
 extern "C" int eng_block_forward(EngPart* block, EngCtx* ctx, const EngMat* h, int cache_slot,
-                                 int writes_cache) {
+                                 int writes_cache, int state_slot) {
   Block* b = as<Block>(block, KIND_BLOCK, "eng_block_forward");
-  return b ? b->forward(ctx, *h, cache_slot, writes_cache != 0) : 1;
+  return b ? b->forward(ctx, *h, cache_slot, writes_cache != 0, state_slot) : 1;
 }
 
 extern "C" int eng_norm_forward(EngPart* norm, EngCtx* ctx, const EngMat* x, const int* rows, int n_rows,

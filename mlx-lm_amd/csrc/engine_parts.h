@@ -54,8 +54,12 @@ struct Position : EngPart {
 // this run puts the step's tokens there.  accepts_lazy: x may be a norm not computed yet
 // (EngHost.materialize computes it); accepts_packed: x may come in the packed order;
 // first_weight: the weights that x meets first, for kernels before it that read ahead.
+// can_overwrite: the part is able to write its output into `residual` instead of adding to it;
+// an arrangement that wants the output by itself (a sum that is normed afterwards) then sets
+// `overwrite` on the parts it owns, and hands the others rows of zeros.
 struct Mixer : EngPart {
   bool accepts_lazy = false, accepts_packed = false;
+  bool can_overwrite = false, overwrite = false;
   const EngWeight* first_weight = nullptr;
   Mixer() : EngPart(KIND_MIXER) {}
   virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) = 0;
@@ -63,15 +67,18 @@ struct Mixer : EngPart {
 
 struct FeedForward : EngPart {
   bool accepts_lazy = false, accepts_packed = false;
+  bool can_overwrite = false, overwrite = false;
   const EngWeight* first_weight = nullptr;
   FeedForward() : EngPart(KIND_FFN) {}
   virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual) = 0;
 };
 
+// `state_slot`: the cache slot of per-request state that the arrangement itself keeps for this
+// run (the row before a portion's first, for a token shift), or -1.
 struct Block : EngPart {
   bool handles_pending = false;
   Block() : EngPart(KIND_BLOCK) {}
-  virtual int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes) = 0;
+  virtual int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int state_slot) = 0;
 };
 
 struct Embedding : EngPart {

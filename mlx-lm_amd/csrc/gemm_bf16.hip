@@ -20,7 +20,8 @@
 #include <algorithm>
 #include <type_traits>
 
-#define FLAG_GELU 1
+#define FLAG_GELU FLAG_ACT_GELU
+#define FLAG_RELU2 FLAG_ACT_RELU2  // the square of the ReLU instead
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
 #define FLAG_KV 8  // columns from q_width on are keys, then values: they go to their cache pages, not to out
@@ -75,7 +76,7 @@ __device__ __forceinline__ uint16_t* kv_place(const GemmArgs& p, int m, int n) {
 
 __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
   if (p.bias) v += p.bias[n];
-  if (p.flags & FLAG_GELU) v = gelu_tanh_fast(v);
+  v = activate<true>(p.flags, v);
   if ((p.flags & FLAG_KV) && n >= p.q_width) {
     *kv_place(p, m, n) = f32_to_bf16_bits(v);
     return;
@@ -463,6 +464,11 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
           for (int s = 0; s < GROUP; ++s)
 #pragma unroll
             for (int c = 0; c < CPL; ++c) v[s][c] = gelu_tanh_fast(v[s][c]);
+        } else if (p.flags & FLAG_RELU2) {
+#pragma unroll
+          for (int s = 0; s < GROUP; ++s)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v[s][c] = relu_squared(v[s][c]);
         }
 #pragma unroll
         for (int s = 0; s < GROUP; ++s) {
@@ -607,8 +613,9 @@ static int check_args(const GemmArgs& p) {
   const size_t w_elements = p.w_packed ? (size_t)((p.N + 15) / 16) * p.w_kblocks * 1024 : (size_t)p.N * p.ldw;
   if ((size_t)p.M * p.lda >= (1u << 31) || w_elements >= (1u << 31))
     FAIL("gemm_bf16: operands of 2^31 elements or more are not supported");
-  if ((p.flags & FLAG_ACCUMULATE) && (p.flags & FLAG_GELU))
-    FAIL("gemm_bf16: GELU and accumulate cannot be combined");
+  if ((p.flags & FLAG_ACCUMULATE) && (p.flags & FLAG_ACT_ANY))
+    FAIL("gemm_bf16: an activation and accumulate cannot be combined");
+  if ((p.flags & FLAG_ACT_ANY) == FLAG_ACT_ANY) FAIL("gemm_bf16: two activations at once");
   return 0;
 }
 
@@ -746,7 +753,7 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
   p.out = out;
   p.M = M, p.N = N, p.K = K;
   p.lda = lda, p.ldw = ldw, p.ldo = ldo;
-  p.flags = flags & (FLAG_GELU | FLAG_ACCUMULATE | FLAG_OUT_F32);
+  p.flags = flags & (FLAG_ACT_ANY | FLAG_ACCUMULATE | FLAG_OUT_F32);
   p.w_packed = ldw == 0 ? 1 : 0, p.w_kblocks = (K + BK - 1) / BK;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
@@ -754,7 +761,7 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
   p.block_table = block_table, p.token_req = token_req, p.positions = positions;
   p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width, p.head_dim = head_dim, p.page_size = page_size;
   if (k_pages) {
-    if (flags & (FLAG_GELU | FLAG_ACCUMULATE | FLAG_OUT_F32)) FAIL("gemm_bf16: the cache scatter goes with a plain bfloat16 output");
+    if (flags & (FLAG_ACT_ANY | FLAG_ACCUMULATE | FLAG_OUT_F32)) FAIL("gemm_bf16: the cache scatter goes with a plain bfloat16 output");
     if (n_splits > 1) FAIL("gemm_bf16: with K split, sum_partials scatters keys and values");
     if (!v_pages || !block_table || !token_req || !positions)
       FAIL("gemm_bf16: the cache scatter needs pages, block table, token_req and positions");

@@ -45,7 +45,8 @@
 
 #include <mutex>
 
-#define FLAG_GELU 1
+#define FLAG_GELU FLAG_ACT_GELU
+#define FLAG_RELU2 FLAG_ACT_RELU2  // the square of the ReLU instead
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
 #define FLAG_KV 8
@@ -103,7 +104,7 @@ struct FinishLoads {
 };
 __device__ __forceinline__ void finish_with(const DecodeGemmArgs& p, int m, int n, float v, const FinishLoads& l) {
   if (p.bias) v += l.bias;
-  if (p.flags & FLAG_GELU) v = gelu_tanh_fast(v);
+  v = activate<true>(p.flags, v);
   if ((p.flags & FLAG_KV) && n >= p.q_width) {
     const int c = n - p.q_width;
     const bool is_v = c >= p.kv_width;
@@ -139,7 +140,8 @@ __device__ __forceinline__ void finish(const DecodeGemmArgs& p, int m, int n, fl
 __device__ __forceinline__ void finish4_with(const DecodeGemmArgs& p, int m, int n, float4 v, const float4& b, int pos,
                                              int page) {
   if (p.bias) v.x += b.x, v.y += b.y, v.z += b.z, v.w += b.w;
-  if (p.flags & FLAG_GELU) v.x = gelu_tanh_fast(v.x), v.y = gelu_tanh_fast(v.y), v.z = gelu_tanh_fast(v.z), v.w = gelu_tanh_fast(v.w);
+  if (p.flags & FLAG_ACT_ANY)
+    v.x = activate<true>(p.flags, v.x), v.y = activate<true>(p.flags, v.y), v.z = activate<true>(p.flags, v.z), v.w = activate<true>(p.flags, v.w);
   uint2 packed;
   packed.x = pack2(v.x, v.y), packed.y = pack2(v.z, v.w);
   if ((p.flags & FLAG_KV) && n >= p.q_width) {
@@ -772,8 +774,9 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
                          const int* positions, int q_width, int kv_width, int head_dim, int page_size) {
   if (N <= 0) FAIL("%s: bad N=%d", who, N);
   if (!out) FAIL("%s: null pointer", who);
-  if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_GELU | FLAG_KV)))
-    FAIL("%s: accumulate cannot be combined with GELU or the cache scatter", who);
+  if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_ACT_ANY | FLAG_KV)))
+    FAIL("%s: accumulate cannot be combined with an activation or the cache scatter", who);
+  if ((flags & FLAG_ACT_ANY) == FLAG_ACT_ANY) FAIL("%s: two activations at once", who);
   if ((flags & FLAG_OUT_PACKED) && (flags & (FLAG_ACCUMULATE | FLAG_OUT_F32 | FLAG_KV)))
     FAIL("%s: the packed order is for a bfloat16 out that is neither added to nor scattered", who);
   if (flags & FLAG_KV) {
@@ -782,7 +785,7 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
     if (head_dim <= 0 || page_size <= 0 || kv_width % head_dim != 0 || q_width + 2 * kv_width != N)
       FAIL("%s: q_width %d + 2 * kv_width %d must be N=%d, kv_width a multiple of head_dim %d", who,
            q_width, kv_width, N, head_dim);
-    if (flags & (FLAG_OUT_F32 | FLAG_GELU)) FAIL("%s: the cache scatter writes bfloat16, no GELU", who);
+    if (flags & (FLAG_OUT_F32 | FLAG_ACT_ANY)) FAIL("%s: the cache scatter writes bfloat16, no activation", who);
     if (ldo < q_width) FAIL("%s: ldo=%d smaller than q_width=%d", who, ldo, q_width);
   } else if (ldo < N && !(flags & FLAG_OUT_PACKED)) {
     FAIL("%s: ldo=%d smaller than N=%d", who, ldo, N);

@@ -14,7 +14,8 @@
 // units, K goes in parts and a second kernel (the caller's) adds them up.
 #include "common.h"
 
-#define FLAG_GELU 1
+#define FLAG_GELU FLAG_ACT_GELU
+#define FLAG_RELU2 FLAG_ACT_RELU2  // the square of the ReLU instead
 #define FLAG_ACCUMULATE 2
 
 struct GemmArgs {
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           v[j][r] = acc[i][j][r] + bias;
-          if (p.flags & FLAG_GELU) v[j][r] = gelu_tanh(v[j][r]);
+          v[j][r] = activate<false>(p.flags, v[j][r]);
         }
       }
     }
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(64 * SKF_MAX_WAVES) void gemm_f32_skinny_kernel(Gem
       if (p.flags & FLAG_ACCUMULATE)
         p.out[idx] += v;
       else
-        p.out[idx] = (p.flags & FLAG_GELU) ? gelu_tanh(v) : v;
+        p.out[idx] = activate<false>(p.flags, v);
     }
   }
 }
@@ -312,8 +313,8 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
     FAIL("gemm_f32: row strides smaller than the rows (lda=%d ldw=%d ldo=%d)", lda, ldw, ldo);
   if (!A || !W || !out) FAIL("gemm_f32: null pointer");
   if (((uintptr_t)A | (uintptr_t)W) & 15) FAIL("gemm_f32: A and W must be 16-byte aligned");
-  if ((flags & FLAG_ACCUMULATE) && (flags & FLAG_GELU))
-    FAIL("gemm_f32: GELU and accumulate cannot be combined");
+  if ((flags & FLAG_ACCUMULATE) && (flags & FLAG_ACT_ANY))
+    FAIL("gemm_f32: an activation and accumulate cannot be combined");
   if (M == 0) return 0;
   if (n_splits < 1) FAIL("gemm_f32: n_splits=%d", n_splits);
   if (n_splits > 1) {

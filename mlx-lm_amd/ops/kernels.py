@@ -106,8 +106,8 @@ def _rows2d(t, name):
 # ---------------------------------------------------------------------------
 
 
-def embed_gather_add(out, table, ids, add_table=None, add_ids=None):
-    """``out[t] = table[ids[t]] (+ add_table[add_ids[t]])`` into float32 ``out``."""
+def embed_gather_add(out, table, ids, add_table=None, add_ids=None, scale=1.0):
+    """``out[t] = table[ids[t]] * scale (+ add_table[add_ids[t]])`` into float32 ``out``."""
     lib = build.load("embed")
     n, width = out.shape
     _dev(out, "out", torch.float32)
@@ -119,9 +119,9 @@ def embed_gather_add(out, table, ids, add_table=None, add_ids=None):
         _dev(add_table, "add_table", table.dtype)
         _dev(add_ids, "add_ids", torch.int32)
         _need(add_table.shape[1] == width and add_ids.numel() >= n, "embed_gather_add: shapes disagree")
-    rc = lib.embed_gather_add(
+    rc = lib.embed_scale_add(
         _ptr(out), _ptr(table), _ptr(ids), _ptr(add_table), _ptr(add_ids),
-        _c_int(n), _c_int(width), _c_int(DT[table.dtype]), _stream(),
+        _c_int(n), _c_int(width), _c_int(DT[table.dtype]), ctypes.c_float(scale), _stream(),
     )
     build.check(lib, rc, "embed_gather_add")
     return out

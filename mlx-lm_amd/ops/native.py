@@ -153,14 +153,14 @@ def lib():
                                    POINTER(EngWeight), P, P, c_int]),
         "eng_make_gelu_mlp": (P, [c_int, c_int, POINTER(EngWeight), P, POINTER(EngWeight), P]),
         "eng_make_pre_norm_block": (P, [P, P, P, P]),
-        "eng_make_token_embedding": (P, [P, c_int, c_int, c_int]),
+        "eng_make_token_embedding": (P, [P, c_int, c_int, c_int, c_float]),
         "eng_make_learned_positions": (P, [P, c_int, c_int, c_int]),
         "eng_make_linear_head": (P, [POINTER(EngWeight)]),
         "eng_make_model": (P, [c_int, c_int, P, P, c_int, POINTER(P), c_int, POINTER(c_int), POINTER(c_int),
-                               POINTER(c_int), P, P]),
+                               POINTER(c_int), POINTER(c_int), P, P]),
         "eng_free": (None, [P]),
         "eng_model_forward": (c_int, [P, POINTER(EngCtx)]),
-        "eng_block_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngMat), c_int, c_int]),
+        "eng_block_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngMat), c_int, c_int, c_int]),
         "eng_norm_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngMat), P, c_int, c_int, POINTER(EngWeight),
                                      POINTER(EngValue)]),
         "eng_mixer_forward": (c_int, [P, POINTER(EngCtx), POINTER(EngValue), POINTER(EngMat), c_int, c_int]),
@@ -210,6 +210,17 @@ def host():
     """The host's table of routines (``EngHost`` of csrc/engine.h), for the maker of a native part
     that lives in a library of its own (csrc/engine_parts.h)."""
     return lib().eng_host()
+
+
+def part_library(name, makers):
+    """The library of a native part that lives in a source of its own (``csrc/<name>.hip``), with
+    the signatures of its makers set: ``makers`` maps a maker's name to the ctypes types of its
+    arguments after the host's table.  Every maker returns the part's handle."""
+    L = build.load(name)
+    for maker, argtypes in makers.items():
+        fn = getattr(L, maker)
+        fn.restype, fn.argtypes = c_void_p, [c_void_p, *argtypes]
+    return L
 
 
 def made(handle, what):

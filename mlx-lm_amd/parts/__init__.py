@@ -1,6 +1,6 @@
 """Parts that models are put together from; importing this registers the built-in kinds."""
 
-from . import attention, block, embedding, feed_forward, head, norms, positions  # noqa: F401
+from . import attention, block, embedding, feed_forward, gated_attention, head, norms, positions  # noqa: F401
 from .base import (
     BLOCKS,
     EMBEDDINGS,

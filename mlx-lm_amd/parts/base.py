@@ -164,6 +164,11 @@ class Block(Part):
     def cache_need(self):
         return None
 
+    def state_need(self):
+        """A ``StateNeed`` for per-request state that the arrangement itself keeps (one slot for
+        each run of the layer, ``RunEntry.state``), or ``None``."""
+        return None
+
     def forward(self, ctx, h, cache, writes_cache=True):
         raise NotImplementedError
 

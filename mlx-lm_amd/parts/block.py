@@ -2,8 +2,9 @@
 
 import ctypes
 
+from ..config.plan import StateNeed
 from ..ops import native
-from .base import Block, register_block
+from .base import Block, TensorSpec, register_block
 
 
 class PreNormBlock(Block):
@@ -40,9 +41,90 @@ class PreNormBlock(Block):
         hm = native.mat(h)
         with ctx.enter():
             rc = native.lib().eng_block_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(hm), cache.slot,
-                                                int(bool(writes_cache)))
+                                                int(bool(writes_cache)), -1)
         native.check(rc, "pre-norm block")
         return h
 
 
+class PostNormBlock(Block):
+    """``h = norm1(alpha h + s1 * mixer(shift(h))); h = norm2(alpha h + s2 * ffn(h))``: the norms
+    come after the sums, and the sublayers read the stream itself.
+
+    ``layer_scale``: the sublayers' outputs are multiplied per column by the tensors ``ls1`` and
+    ``ls2`` before they enter the sums.  ``token_shift``: the mixer reads ``h_t + (h_{t-1} - h_t) *
+    shift`` per column (zeros before a request's first token); the row before a portion's first
+    is per-request state that the arrangement keeps, one slot for each run of the layer
+    (``state_need``).  The feed-forward (with its norm) may be absent.  Both norms are RMS norms
+    (``rmsnorm`` parts give weight and eps); sums, scales, shift and norms run in float32 in the
+    arrangement's own kernels (csrc/post_norm_block.hip).  No counterpart in
+    mlx_lm/models/gpt2.py, whose blocks norm before their sublayers (:98-108).
+    """
+
+    PARTS = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "feed_forward", "ffn_norm": "norm"}
+    OPTIONAL = ("ffn", "ffn_norm")
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, mixer, mixer_norm, ffn=None, ffn_norm=None, alpha=1.0, layer_scale=False, token_shift=False,
+                 scale_names=("ls1", "ls2"), shift_name="shift", prefix=""):
+        super().__init__(prefix)
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a post-norm layer has a feed-forward and its norm, or neither")
+        for norm in (mixer_norm, ffn_norm):
+            if norm is not None and not (hasattr(norm, "weight") and hasattr(norm, "eps") and not hasattr(norm, "bias")):
+                raise ValueError(f"the post-norm arrangement fuses RMS norms, not a {type(norm).__name__}")
+        if ffn_norm is not None and (ffn_norm.eps != mixer_norm.eps or ffn_norm.width != mixer_norm.width):
+            raise ValueError("the two norms of a post-norm layer share width and eps")
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+        self.width, self.alpha = mixer_norm.width, float(alpha)
+        self.layer_scale, self.token_shift = bool(layer_scale), bool(token_shift)
+        self.scale_names, self.shift_name = tuple(self._name(n) for n in scale_names), self._name(shift_name)
+        self.scale1 = self.scale2 = self.shift = None
+
+    def parts(self):
+        # (the arrangement owns tensors itself, so it is one of its own parts)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self) if p is not None)
+
+    def tensors(self):
+        t = {}
+        if self.layer_scale:
+            t[self.scale_names[0]] = TensorSpec((self.width,), "vector")
+            if self.ffn is not None:
+                t[self.scale_names[1]] = TensorSpec((self.width,), "vector")
+        if self.token_shift:
+            t[self.shift_name] = TensorSpec((self.width,), "vector")
+        return t
+
+    def load(self, tensors):
+        if self.layer_scale:
+            self.scale1 = tensors[self.scale_names[0]]
+            self.scale2 = tensors[self.scale_names[1]] if self.ffn is not None else None
+        if self.token_shift:
+            self.shift = tensors[self.shift_name]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def state_need(self):
+        return StateNeed((self.width,), "float32") if self.token_shift else None
+
+    def make_native(self):
+        P, F = ctypes.c_void_p, ctypes.c_float
+        L = native.part_library("post_norm_block", {"make_post_norm_block": [P, P, ctypes.c_int, F, F, P, P, P, P, P]})
+        return native.made(L.make_post_norm_block(
+            native.host(), self.mixer.native(), self.ffn.native() if self.ffn is not None else None, self.width,
+            self.alpha, self.mixer_norm.eps, native.ptr(self.mixer_norm.weight),
+            native.ptr(self.ffn_norm.weight) if self.ffn_norm is not None else None, native.ptr(self.scale1),
+            native.ptr(self.scale2), native.ptr(self.shift)), "post-norm block")
+
+    def forward(self, ctx, h, cache, writes_cache=True, state=None):
+        """``state``: the ``CacheView`` of the run's state slot (with ``token_shift``)."""
+        hm = native.mat(h)
+        with ctx.enter():
+            rc = native.lib().eng_block_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(hm), cache.slot,
+                                                int(bool(writes_cache)), state.slot if state is not None else -1)
+        native.check(rc, "post-norm block")
+        return h
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("post_norm", PostNormBlock)

@@ -5,15 +5,16 @@ from .base import Part, TensorSpec, register_embedding
 
 
 class TokenEmbedding(Part):
-    """``h[t] = table[ids[t]]``, plus a position term if the model has one.
+    """``h[t] = table[ids[t]] * scale``, plus a position term (not scaled) if the model has one.
 
-    mlx_lm/models/gpt2.py:119-120,132.
+    mlx_lm/models/gpt2.py:119-120,132 (where ``scale`` is 1).
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
 
-    def __init__(self, vocab_size, width, weight_name="weight", prefix=""):
+    def __init__(self, vocab_size, width, weight_name="weight", scale=1.0, prefix=""):
         super().__init__(prefix)
+        self.scale = float(scale)
         if vocab_size <= 0 or width <= 0:
             raise ValueError(f"embedding sizes must be positive, got {vocab_size} x {width}")
         self.vocab_size, self.width = vocab_size, width
@@ -34,14 +35,14 @@ class TokenEmbedding(Part):
 
     def make_native(self):
         return native.made(native.lib().eng_make_token_embedding(
-            self.table.data_ptr(), self.vocab_size, self.width, native.DT[self.table.dtype]), "token embedding")
+            self.table.data_ptr(), self.vocab_size, self.width, native.DT[self.table.dtype], self.scale), "token embedding")
 
     def forward(self, ctx, out, add=None):
         """Fill float32 ``out [tokens, width]``; ``add`` is ``(table, index)`` or ``None``."""
         if add is None:
-            kernels.embed_gather_add(out, self.table, ctx.token_ids)
+            kernels.embed_gather_add(out, self.table, ctx.token_ids, scale=self.scale)
         else:
-            kernels.embed_gather_add(out, self.table, ctx.token_ids, add[0], add[1])
+            kernels.embed_gather_add(out, self.table, ctx.token_ids, add[0], add[1], scale=self.scale)
         return out
 
 

@@ -70,4 +70,53 @@ class GeluMLP(FeedForward):
         native.check(rc, "gelu_mlp")
 
 
+class Relu2MLP(FeedForward):
+    """``down(relu(up(x))^2)``, dense, no biases.
+
+    The activation is fused into the first product.  The second adds into ``residual``, or, in an
+    arrangement that wants the output by itself (``post_norm``), writes it there.  No counterpart
+    in mlx_lm/models/gpt2.py, whose MLP is the tanh GELU's.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, inner, up_name="up", down_name="down", prefix=""):
+        super().__init__(prefix)
+        if width % 8:
+            raise ValueError(f"the feed-forward's width must be a multiple of 8, got {width}")
+        if inner <= 0:
+            raise ValueError(f"the feed-forward's inner size must be positive, got {inner}")
+        self.width, self.inner = width, inner
+        self.inner_padded = (inner + 7) // 8 * 8  # zero weights beyond ``inner``: relu(0)^2 = 0 meets zero columns
+        self.up_name, self.down_name = self._name(up_name), self._name(down_name)
+        self.up_w = self.down_w = None
+
+    def tensors(self):
+        return {self.up_name: TensorSpec((self.inner, self.width), "matrix"),
+                self.down_name: TensorSpec((self.width, self.inner), "matrix")}
+
+    def load(self, tensors):
+        up, down = tensors[self.up_name], tensors[self.down_name]
+        pad = self.inner_padded - self.inner
+        if pad:
+            up = torch.cat([up, up.new_zeros(pad, self.width)]).contiguous()
+            down = torch.cat([down, down.new_zeros(self.width, pad)], dim=1).contiguous()
+        self.up_w, self.down_w = kernels.for_decode(up), kernels.for_decode(down)
+        self.first_weight = self.up_w
+
+    def make_native(self):
+        W = ctypes.POINTER(native.EngWeight)
+        L = native.part_library("relu2_mlp", {"make_relu2_mlp": [ctypes.c_int, ctypes.c_int, W, W]})
+        up_w, down_w = kernels.weight_struct(self.up_w), kernels.weight_struct(self.down_w)
+        return native.made(L.make_relu2_mlp(native.host(), self.width, self.inner_padded, ctypes.byref(up_w),
+                                            ctypes.byref(down_w)), "relu2_mlp")
+
+    def forward(self, ctx, x, residual):
+        v, r = value_of(x), native.mat(residual)
+        with ctx.enter():
+            rc = native.lib().eng_ffn_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(v), ctypes.byref(r))
+        native.check(rc, "relu2_mlp")
+
+
 register_feed_forward("gelu_mlp", GeluMLP)
+register_feed_forward("relu2_mlp", Relu2MLP)

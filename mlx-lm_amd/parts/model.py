@@ -35,12 +35,12 @@ class DecoderModel:
                     f"unknown block arrangement '{spec.arrangement}' (known: {sorted(BLOCKS)})"
                 )
             cls = BLOCKS[spec.arrangement]
-            if set(spec.parts) != set(cls.PARTS):
+            if not (set(cls.PARTS) - set(getattr(cls, "OPTIONAL", ())) <= set(spec.parts) <= set(cls.PARTS)):
                 raise ValueError(
                     f"arrangement '{spec.arrangement}' arranges {sorted(cls.PARTS)}, the plan gives {sorted(spec.parts)}"
                 )
             built = {name: build_part(*FAMILIES[cls.PARTS[name]], part_spec) for name, part_spec in spec.parts.items()}
-            self.layers.append(cls(**built))
+            self.layers.append(cls(**built, **getattr(spec, "params", {})))
         self.schedule = list(plan.schedule)
         self.final_norm = build_part(NORMS, "norm", plan.final_norm)
         self.head = build_part(HEADS, "output head", plan.head)
@@ -109,6 +109,13 @@ class DecoderModel:
                     f"layer {run.layer} reads cache slot {run.cache} but wants {need}, "
                     f"the slot holds {needs[run.cache]}"
                 )
+        for run in self.schedule:
+            block = self.layers[run.layer]
+            need = block.state_need() if hasattr(block, "state_need") else None
+            if (need is None) != (run.state is None):
+                raise ValueError(f"layer {run.layer} {'keeps state of its own: its runs need a state slot' if need else 'keeps no state of its own, but its run names a state slot'}")
+            if need is not None:
+                needs[run.state] = need
         out = [needs[i] for i in range(len(needs))]
         for need in out:
             if need is not None and not isinstance(need, (CacheNeed, StateNeed)):
@@ -144,6 +151,7 @@ class DecoderModel:
                 self.embedding_positions.native() if self.embedding_positions is not None else None,
                 len(self.layers), layers, n, ints(*[r.layer for r in self.schedule]),
                 ints(*[r.cache for r in self.schedule]), ints(*[int(r.writes_cache) for r in self.schedule]),
+                ints(*[-1 if r.state is None else r.state for r in self.schedule]),
                 self.final_norm.native(), self.head.native()), "model")
         return self._native
 

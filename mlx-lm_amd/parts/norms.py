@@ -56,4 +56,44 @@ class LayerNorm(Norm):
         return ctx.tensor(out.m)
 
 
+class RMSNorm(Norm):
+    """``x / sqrt(mean(x^2) + eps) * weight``: no mean is taken off, eps sits inside the root.
+
+    Reads the float32 residual stream, computes in float32, writes the compute dtype (``rows``:
+    only those rows, for the rows whose logits are wanted).  An arrangement that norms after
+    its sums (``post_norm``) takes ``weight`` and ``eps`` from here and fuses the norm into its
+    own kernel.  No counterpart in mlx_lm/models/gpt2.py, whose norms are LayerNorms.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, width, eps, weight_name="weight", prefix=""):
+        super().__init__(prefix)
+        if eps < 0:
+            raise ValueError(f"eps must not be negative, got {eps}")
+        self.width, self.eps = width, float(eps)
+        self.weight_name = self._name(weight_name)
+        self.weight = None
+
+    def tensors(self):
+        return {self.weight_name: TensorSpec((self.width,), "vector")}
+
+    def load(self, tensors):
+        self.weight = tensors[self.weight_name]
+
+    def make_native(self):
+        L = native.part_library("rmsnorm", {"make_rmsnorm": [ctypes.c_int, ctypes.c_float, ctypes.c_void_p]})
+        return native.made(L.make_rmsnorm(native.host(), self.width, self.eps, native.ptr(self.weight)), "rmsnorm")
+
+    def forward(self, ctx, x, rows=None, n_rows=None, lazy=False):
+        out = native.EngValue()
+        xm = native.mat(x)
+        with ctx.enter():
+            rc = native.lib().eng_norm_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(xm), native.ptr(rows),
+                                               int(n_rows or 0), 0, None, ctypes.byref(out))
+        native.check(rc, "rmsnorm")
+        return ctx.tensor(out.m)
+
+
 register_norm("layernorm", LayerNorm)
+register_norm("rmsnorm", RMSNorm)
