@@ -437,9 +437,15 @@ def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out, ahead=None):
     return out
 
 
+ACTIVATIONS = {None: 0, "gelu_tanh": 1, "relu2": 2}  # the product kernels' epilogue activations, by code
+
+
 def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None, splits=None,
-           pending=None):
+           pending=None, activation=None):
     """``out = epilogue(a @ w.T + bias)``.
+
+    ``gelu`` asks for the tanh GELU in the epilogue; ``activation`` names any of ``ACTIVATIONS``
+    (``"relu2"``: the square of the ReLU) instead.
 
     ``a`` is ``[M, K]`` (or a ``NormedInput``), ``w`` is ``[N, K]`` (or a
     ``PackedWeight``, whose packed copy the decode kernel reads), both
@@ -494,7 +500,10 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
                                scatter.token_req.data_ptr(), scatter.positions.data_ptr(),
                                scatter.block_table.shape[1], scatter.q_width, scatter.kv_width, 0)
         call.scatter = ctypes.pointer(sc)
-    call.gelu, call.accumulate, call.variant, call.splits = int(gelu), int(accumulate), int(variant), int(splits or 0)
+    if activation not in ACTIVATIONS:
+        _fail(f"linear: unknown activation {activation!r} (known: {sorted(k for k in ACTIVATIONS if k)})")
+    code = ACTIVATIONS[activation] or int(bool(gelu))
+    call.gelu, call.accumulate, call.variant, call.splits = code, int(accumulate), int(variant), int(splits or 0)
     rc = L.eng_linear(ctypes.byref(ctx), ctypes.byref(call), ctypes.byref(pending.c) if pending is not None else None)
     native.check(rc, "linear")
     return out

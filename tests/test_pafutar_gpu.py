@@ -1,0 +1,402 @@
+"""Pafutar in the engine against the plain implementation (plain_pafutar.py): each mechanism,
+whole prompts, decoding, portions, mixed batches, reused pages, window and kept-first edges,
+generation through the entry points."""
+
+import copy
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_pafutar as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# max |engine - plain| over max |plain logits|: float32 sums where the plain side has float64;
+# bfloat16 rounds activations between the products (the plain side gets the rounded matrices)
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+
+
+def _mixer(heads, kv_heads, dim, window=None, keep_first=0, scale=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale or dim**-0.5}
+    if window is not None:
+        m["mask"] = {"size": window, "keep_first": keep_first}
+    return m
+
+
+def _layer(mixer, ff=None, weights_of=None):
+    e = {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+    if weights_of is not None:
+        e["weights_of"] = weights_of
+    return e
+
+
+def _config(width, vocab, layers, max_positions=256, alpha=1.0, scale=1.0, eps=1e-6):
+    return {"architecture": "Pafutar", "vocab": vocab, "width": width, "max_positions": max_positions,
+            "embedding": {"scale": scale}, "norm": {"eps": eps}, "postln_alpha": alpha, "layers": layers}
+
+
+_A0 = _mixer(4, 2, 16, window=24, keep_first=5, scale=0.3)
+_A1 = _mixer(2, 1, 32, window=40, keep_first=0)
+_B0 = _mixer(3, 3, 48)  # no mask at all
+_B2 = _mixer(2, 2, 24, window=17, keep_first=3)  # a head size that is a multiple of 8 only; edges off the pages' borders
+CONFIGS = {
+    # a layer run twice (with a cache and shift state of its own each), a layer without feed-forward
+    "A": _config(64, 130, [_layer(_A0, 72), _layer(_A1), _layer(_A0, 72, weights_of=0)], alpha=1.7, scale=3.0, eps=1e-5),
+    # no window, an inner size that is no multiple of 8, alpha 1 (the plain sum), kept tokens beyond a page
+    "B": _config(96, 211, [_layer(_B0, 100), _layer(_B2, 52), _layer(_B0, 100, weights_of=0),
+                           _layer(_mixer(4, 1, 16, window=33, keep_first=18), 40)], alpha=1.0, scale=9.5),
+    # head sizes of 64 and 128 (the kernels that stream keys through registers and the matrix cores)
+    "F": _config(128, 300, [_layer(_mixer(2, 1, 64, window=70, keep_first=9), 256), _layer(_mixer(2, 2, 128, window=50, keep_first=33), 128),
+                            _layer(_mixer(4, 2, 32), 64)], max_positions=512, alpha=2.0, scale=11.0),
+}
+SEEDS = {"A": 3, "B": 4, "F": 5}
+
+
+def _folder(path, config, weights):
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    json.dump(config, open(os.path.join(path, "config.json"), "w"))
+    save_file({k: v.contiguous() for k, v in weights.items()}, os.path.join(path, "model.safetensors"))
+    return path
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, config in CONFIGS.items():
+        weights = plain.random_weights(config, SEEDS[name], sharp=4.0)
+        out[name] = (_folder(str(tmp_path_factory.mktemp("paf" + name)), config, weights), config, weights)
+    return out
+
+
+def _engine(folder, dtype, n_pages, page_size=16, max_requests=4, **kw):
+    from mlx_lm_amd.engine import Engine
+    from mlx_lm_amd.utils import load_model
+
+    model, _ = load_model(folder, dtype=dtype)
+    return Engine(model, dtype=dtype, page_size=page_size, n_pages=n_pages, max_requests=max_requests, **kw)
+
+
+def _plain(weights, config, tokens, dtype):
+    w = helpers.round_matrices_to_bf16(weights) if dtype == "bfloat16" else weights
+    return plain.forward(w, config, tokens)
+
+
+def _close(got, want, dtype, what=""):
+    scale = want.abs().max().item()
+    err = (got.double().cpu() - want).abs().max().item()
+    assert err <= TOL[dtype] * scale, f"{what}: max error {err:.3e} against scale {scale:.3e}"
+
+
+def _run(engine, rid, tokens, cuts):
+    from mlx_lm_amd.engine import StepEntry
+
+    engine.add_request(rid)
+    rows, i = [], 0
+    for n in cuts:
+        part = tokens[i : i + n]
+        rows.append(engine.step([StepEntry(rid, part, list(range(len(part))))]).clone())
+        i += n
+    assert i == len(tokens)
+    engine.end_request(rid)
+    return torch.cat(rows)
+
+
+# -- each mechanism alone ------------------------------------------------------------
+
+
+def _ctypes_lib(name):
+    from mlx_lm_amd.ops import build
+
+    return build.load(name)
+
+
+def _stream():
+    from mlx_lm_amd.ops import kernels
+
+    return kernels._stream()
+
+
+@pytest.mark.parametrize("width", [64, 100, 333])
+def test_rmsnorm_kernel(width):
+    import ctypes
+
+    L = _ctypes_lib("rmsnorm")
+    g = torch.Generator().manual_seed(width)
+    x = (torch.randn(9, width, generator=g) * 3).cuda()
+    gamma = (1 + 0.3 * torch.randn(width, generator=g)).cuda()
+    rows = torch.tensor([7, 0, 3], dtype=torch.int32).cuda()
+    for dtype, code, tol in ((torch.float32, 0, 1e-6), (torch.bfloat16, 1, 1e-2)):
+        out = torch.empty(3, width, dtype=dtype, device="cuda")
+        rc = L.rmsnorm(ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(x.data_ptr()), width, ctypes.c_void_p(rows.data_ptr()),
+                       ctypes.c_void_p(gamma.data_ptr()), ctypes.c_float(1e-3), 3, width, code, _stream())
+        assert rc == 0, L.mlxlm_last_error()
+        want = plain.rms_norm(x.double().cpu()[[7, 0, 3]], gamma.double().cpu(), 1e-3)
+        assert (out.double().cpu() - want).abs().max() <= tol * want.abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_token_shift_and_the_sum_that_is_normed(dtype):
+    """Two requests' rows side by side: the shift reads the row before (the state for a portion's
+    first row), the fused sum-and-norm keeps each request's last old row in the state."""
+    import ctypes
+
+    L = _ctypes_lib("post_norm_block")
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    W, g = 72, torch.Generator().manual_seed(1)
+    h = torch.randn(7, W, generator=g).cuda()
+    mu, s, gamma = (torch.rand(W, generator=g).cuda() for _ in range(3))
+    state = torch.randn(4, W, generator=g).cuda()
+    slot_ids = torch.tensor([2, 0], dtype=torch.int32).cuda()
+    token_req = torch.tensor([0, 0, 0, 1, 1, 1, 1], dtype=torch.int32).cuda()
+    code = 0 if dtype == torch.float32 else 1
+    out = torch.empty(7, W, dtype=dtype, device="cuda")
+    assert L.token_shift(P(out), P(h), W, P(mu), P(state), ctypes.c_size_t(W), P(slot_ids), P(token_req), 7, W, code, _stream()) == 0
+    hc, sc = h.double().cpu(), state.double().cpu()
+    want = torch.cat([plain.token_shift(hc[:3], mu.double().cpu(), sc[2]), plain.token_shift(hc[3:], mu.double().cpu(), sc[0])])
+    assert (out.double().cpu() - want).abs().max() <= (1e-6 if code == 0 else 2e-2)
+    y = torch.randn(7, W, generator=g).cuda()
+    copy_ = torch.empty(7, W, dtype=dtype, device="cuda")
+    h2 = h.clone()
+    assert L.residual_rmsnorm(P(h2), W, P(y), W, ctypes.c_float(1.5), P(s), P(gamma), ctypes.c_float(1e-4), P(state),
+                              ctypes.c_size_t(W), P(slot_ids), P(token_req), P(copy_), code, 7, W, _stream()) == 0
+    want = plain.rms_norm(1.5 * hc + s.double().cpu() * y.double().cpu(), gamma.double().cpu(), 1e-4)
+    assert (h2.double().cpu() - want).abs().max() <= 2e-6
+    assert (copy_.double().cpu() - want).abs().max() <= (2e-6 if code == 0 else 2e-2)
+    assert torch.equal(state[2], h[2]) and torch.equal(state[0], h[6])  # the old rows, not the normed ones
+    assert torch.equal(state[1].cpu(), sc[1].float()) and torch.equal(state[3].cpu(), sc[3].float())
+
+
+@pytest.mark.parametrize("rows", [3, 40, 200])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_squared_relu_in_the_products_epilogue(rows, dtype):
+    from mlx_lm_amd.ops import kernels
+
+    g = torch.Generator().manual_seed(rows)
+    a = torch.randn(rows, 96, generator=g).to(dtype).cuda()
+    w = (torch.randn(136, 96, generator=g) * 0.2).to(dtype).cuda()
+    out = torch.empty(rows, 136, dtype=dtype, device="cuda")
+    kernels.linear(out, a, kernels.for_decode(w), activation="relu2")
+    want = torch.relu(a.double().cpu() @ w.double().cpu().t()) ** 2
+    assert (out.double().cpu() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
+    with pytest.raises(ValueError, match="activation"):
+        kernels.linear(out, a, w, activation="swish")
+
+
+def test_the_mixer_alone_and_the_feed_forward_alone(tmp_path):
+    """One layer without feed-forward (the mixer with shift, scale and norm), and the same with
+    one: the difference is the feed-forward's half."""
+    for ff in (None, 48):
+        config = _config(64, 90, [_layer(_mixer(2, 1, 32, window=12, keep_first=2), ff)], alpha=0.5, scale=2.0)
+        weights = plain.random_weights(config, 11, sharp=3.0)
+        folder = _folder(str(tmp_path / f"ff{ff}"), config, weights)
+        tokens = helpers.random_tokens(60, 90, seed=2)
+        got = _run(_engine(folder, "float32", 8), "r", tokens, [60])
+        _close(got, plain.forward(weights, config, tokens), "float32", f"one layer, ff={ff}")
+
+
+# -- the tests' weights show what they are meant to show ---------------------------------
+
+
+@pytest.mark.parametrize("name", ["A", "B", "F"])
+def test_the_plain_side_notices_a_window_a_kept_token_and_a_shift(models, name):
+    """With these weights a window one token off, a kept token left out or a missing shift move
+    the logits by hundreds of times the float32 tolerance: the comparisons below would show them."""
+    _, config, weights = models[name]
+    tokens = helpers.random_tokens(120, config["vocab"], seed=1)
+    base = plain.forward(weights, config, tokens)
+    scale = base.abs().max().item()
+
+    def moved(change):
+        c, w = copy.deepcopy(config), dict(weights)
+        change(c, w)
+        return (plain.forward(w, c, tokens) - base)[60:].abs().max().item() / scale
+
+    def window(c, w):
+        for entry in c["layers"]:
+            if "mask" in entry["mixer"]:
+                entry["mixer"]["mask"]["size"] += 1
+
+    def kept(c, w):
+        for entry in c["layers"]:
+            if entry["mixer"].get("mask", {}).get("keep_first", 0) > 0:
+                entry["mixer"]["mask"]["keep_first"] -= 1
+
+    def shift(c, w):
+        w["l0.shift"] = torch.zeros_like(w["l0.shift"])
+
+    for change in (window, kept, shift):
+        assert moved(change) > 300 * TOL["float32"], change.__name__
+
+
+# -- whole, decoded, portions ----------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n", [("A", 200), ("B", 150), ("F", 300)])
+def test_whole_decoded_and_portions(models, dtype, name, n):
+    folder, config, weights = models[name]
+    tokens = helpers.random_tokens(n, config["vocab"], seed=n)
+    want = _plain(weights, config, tokens, dtype)
+    eng = _engine(folder, dtype, n_pages=(n + 15) // 16 + 2)
+    _close(_run(eng, "whole", tokens, [n]), want, dtype, "whole")
+    # most of it at once, then token by token until every window has passed over decoded tokens
+    _close(_run(eng, "decoded", tokens, [n - 90] + [1] * 90), want, dtype, "last 90 one by one")
+    _close(_run(eng, "portions", tokens, helpers.cuts_changing(n)), want, dtype, "portions of changing size")
+    _close(_run(eng, "twos", tokens[:64], [2] * 32), want[:64], dtype, "portions of two tokens")
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decode(models, dtype):
+    """Every token one by one from the first, up to the model's last position (recorded decode
+    steps replayed, the window and the kept first tokens passing page borders)."""
+    folder, config, weights = models["A"]
+    n = config["max_positions"]
+    tokens = helpers.random_tokens(n, config["vocab"], seed=77)
+    want = _plain(weights, config, tokens, dtype)
+    eng = _engine(folder, dtype, n_pages=n // 16)
+    got = _run(eng, "r", tokens, [1] * n)
+    _close(got[:8], want[:8], dtype, "first tokens")
+    _close(got, want, dtype, "decoding every token")
+
+
+@pytest.mark.parametrize("page_size", [16, 32])
+def test_windows_give_pages_back_and_stale_pages_do_not_matter(models, page_size):
+    """A pool too small for the whole sequence: the windows' passed pages are used again (the kept
+    first tokens' never), and what freed pages hold is never read."""
+    folder, config, weights = models["A"]
+    n = 250
+    tokens = helpers.random_tokens(n, config["vocab"], seed=5)
+    want = _plain(weights, config, tokens, "float32")
+    # the widest window is 40 and 5 tokens are kept: far fewer pages than 250 tokens' worth
+    eng = _engine(folder, "float32", n_pages=8 * 16 // page_size, page_size=page_size)
+    from mlx_lm_amd.engine import StepEntry
+
+    eng.add_request("r")
+    rows, i = [], 0
+    for c in [30, 2, 17] + [1] * 60 + [9, 20, 11] + [1] * 100:
+        rows.append(eng.step([StepEntry("r", tokens[i : i + c], list(range(c)))]).clone())
+        i += c
+        eng.cache.poison_free_pages()
+    assert i == n
+    _close(torch.cat(rows), want, "float32", "a pool smaller than the sequence")
+    rc = eng.cache.requests["r"]
+    for gi, g in enumerate(eng.cache.groups):
+        kept_blocks = (g.need.keep_first + page_size - 1) // page_size
+        assert all(p >= 0 for p in rc.blocks[gi][:kept_blocks])
+        assert any(p < 0 for p in rc.blocks[gi])
+    eng.end_request("r")
+    eng.cache.check()
+
+
+# -- batches -------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "F"])
+def test_mixed_batches_equal_each_request_alone(models, dtype, name):
+    """Up to four live requests of unequal lengths, portions beside single tokens, requests that
+    sit a step out; slots and pages of finished requests are used again by later ones."""
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, weights = models[name]
+    lengths = [70, 9, 131, 40, 3, 97, 55]
+    cfg = {"vocab_size": config["vocab"]}
+    tokens, steps = helpers.mixed_trace(cfg, 21, lengths, n_live=4)
+    eng = _engine(folder, dtype, n_pages=helpers.held(lengths, 4) // 16, max_requests=4)
+    got = {rid: [] for rid in tokens}
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if not eng.has_request(e["id"]):
+                eng.add_request(e["id"])
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        logits = eng.step(entries).clone()
+        at = 0
+        for e in entries:
+            got[e.request_id].append(logits[at : at + len(e.want)])
+            at += len(e.want)
+        for rid in s["end"]:
+            eng.end_request(rid)
+        eng.cache.poison_free_pages()
+    for rid, toks in tokens.items():
+        _close(torch.cat(got[rid]), _plain(weights, config, toks, dtype), dtype, f"request {rid} in mixed batches")
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.n_pages
+
+
+def test_recorded_steps_equal_eager_steps(models):
+    """Decode steps replayed from recorded graphs against the same steps run eagerly, bit for bit
+    (the shift's state is read and written once a step either way)."""
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, _ = models["A"]
+    seqs = {"a": helpers.random_tokens(60, config["vocab"], 1), "b": helpers.random_tokens(45, config["vocab"], 2)}
+    results = {}
+    for use_graphs in (True, False):
+        eng = _engine(folder, "bfloat16", n_pages=10, use_graphs=use_graphs)
+        assert eng.use_graphs == use_graphs  # every part launches kernels only
+        for r in seqs:
+            eng.add_request(r)
+        out = [eng.step([StepEntry("a", seqs["a"][:20], [19]), StepEntry("b", seqs["b"][:5], [4])]).clone()]
+        for i in range(40):
+            out.append(eng.step([StepEntry("a", [seqs["a"][20 + i]], [0]), StepEntry("b", [seqs["b"][5 + i]], [0])]).clone())
+        if use_graphs:
+            assert helpers.decode_graphs(eng, 2)[0].graph is not None
+        results[use_graphs] = torch.cat(out)
+    assert torch.equal(results[True], results[False])
+
+
+# -- generation through the entry points -----------------------------------------------------
+
+
+def _greedy(weights, config, prompt, n):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(plain.forward(weights, config, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+def test_greedy_generation_through_the_scheduler(models):
+    from mlx_lm_amd import batch_generate, load, stream_generate
+
+    folder, config, weights = models["B"]
+    model, tok = load(folder, dtype="float32")
+    prompts = [helpers.random_tokens(n, config["vocab"], seed=n) for n in (23, 5, 61)]
+    want = [_greedy(weights, config, p, 10) for p in prompts]
+    got = [r.token for r in stream_generate(model, tok, prompts[0], max_tokens=10, prefill_step_size=7)]
+    assert got == want[0]
+    batch = batch_generate(model, tok, prompts, max_tokens=10)
+    assert [[int(t) for t in text.split()] for text in batch.texts] == want
+
+
+def test_trace_replay_of_a_random_model(tmp_path, models):
+    """The replay program on a configuration with seeded random weights: logits files per step."""
+    _, config, _ = models["A"]
+    json.dump(config, open(tmp_path / "config.json", "w"))
+    tokens = helpers.random_tokens(50, config["vocab"], seed=9)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": tokens[:31], "want": [30]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": tokens[31:], "want": "all"}], "end": ["x"]}]
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--config", str(tmp_path / "config.json"),
+                           "--seed", "4", "--dtype", "float32", "--out", str(out), "--max-tokens", "64"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "done 0" in proc.stdout and "done 1" in proc.stdout
+    from mlx_lm_amd.config.registry import get_model_classes
+
+    model_cls, args_cls = get_model_classes(config)
+    weights = model_cls.random_weights(args_cls.from_dict(config), 4, "b")
+    want = plain.forward(weights, config, tokens)
+    got = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, config["vocab"])
+    _close(torch.from_numpy(got), want[31:], "float32", "the replay's second step")
