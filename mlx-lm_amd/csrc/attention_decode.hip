@@ -53,7 +53,26 @@ struct DecodeArgs {
   // last at the (row, head)'s counter adds them in the order of the parts (no second kernel);
   // 2: n_splits is the most a row takes, and a row takes as many as its own length calls for
   int join_here;
+  // Optional terms (all absent: plain causal attention), as in attention.hip's AttnArgs:
+  // head_scale [n_heads] instead of `scale`; slopes [n_heads], slope * distance taken off a score;
+  // keep_first, the first keys that a window leaves visible; gate (rows of stride ldg, the
+  // kernel's element type), the output times its sigmoid.
+  const float* head_scale;
+  const float* slopes;
+  const void* gate;
+  int ldg, keep_first;
 };
+
+template <typename T>
+__device__ __forceinline__ float gate_at(const DecodeArgs& p, int row, int col) {
+  if (!p.gate) return 1.f;
+  float g;
+  if (sizeof(T) == 2)
+    g = bits_to_f32(((const uint16_t*)p.gate)[(size_t)row * p.ldg + col]);
+  else
+    g = ((const float*)p.gate)[(size_t)row * p.ldg + col];
+  return 1.0f / (1.0f + expf(-g));
+}
 
 #define MAX_WAVES 16
 
@@ -171,20 +190,25 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   {
     const uint4 qv = *(const uint4*)((const T*)p.q + (size_t)row * p.ldq + h * HD + sub * EPL);
     unpack(qv, qf, (const T*)nullptr);
+    const float q_scale = p.head_scale ? p.head_scale[h] : p.scale;
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) qf[i] *= p.scale;
+    for (int i = 0; i < EPL; ++i) qf[i] *= q_scale;
   }
+  const float slope = p.slopes ? p.slopes[h] : 0.f;
 
   const int k_hi = pos + 1;
   const int k_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
   const int kt0 = (k_lo / TILE) * TILE;
-  const int n_tiles = (k_hi - kt0 + TILE - 1) / TILE;
+  // the kept first keys [0, sink_hi) that the window has left behind come first, in tiles of their own
+  const int sink_hi = min(p.keep_first, k_lo);
+  const int n_sink_tiles = (sink_hi + TILE - 1) / TILE;
+  const int n_tiles = n_sink_tiles + (k_hi - kt0 + TILE - 1) / TILE;
   // Joined here, a row may take fewer splits than the launch has: as many as leave a wave a tile
   // of 32 keys, and one if a wave has fewer than 96 keys anyway (joining costs about a tile's
   // time).  Blocks of the splits it does not take have nothing to do.
   int n_splits = p.n_splits;
   if (p.join_here == 2) {
-    const int keys_a_wave = (k_hi - kt0) / n_waves;
+    const int keys_a_wave = (k_hi - kt0 + n_sink_tiles * TILE) / n_waves;
     n_splits = keys_a_wave >= 96 ? min(n_splits, keys_a_wave / 32) : 1;
     if (split >= n_splits) return;  // (the whole block)
   }
@@ -200,14 +224,16 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   if (p.table_in_lds) __syncthreads();  // (uniform over the block)
 
   for (int t = t_begin + wave; t < t_end; t += n_waves) {
-    const int kt = kt0 + t * TILE;
+    const bool sink = t < n_sink_tiles;
+    const int kt = sink ? t * TILE : kt0 + (t - n_sink_tiles) * TILE;
+    const int t_lo = sink ? 0 : k_lo, t_hi = sink ? sink_hi : k_hi;  // the run of keys this tile is of
     uint4 kv[NL], vv[NL];
-    // all loads of the tile first; addresses of keys outside [k_lo, k_hi) are
+    // all loads of the tile first; addresses of keys outside the run are
     // pulled inside (their scores are masked below)
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
       int key = kt + j * KPL + kin;
-      key = min(max(key, k_lo), k_hi - 1);
+      key = min(max(key, t_lo), t_hi - 1);
       const int page = p.table_in_lds ? page_of[key / p.page_size] : table[key / p.page_size];
       const size_t off = (size_t)page * p.page_stride + head_off +
                          (size_t)(key % p.page_size) * HD + sub * EPL;
@@ -225,7 +251,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
       for (int i = 0; i < EPL; ++i) d += qf[i] * kf[i];
       d = group_sum<CPK>(d);  // over the key's lanes
       const int key = kt + j * KPL + kin;
-      s[j] = (key >= k_lo && key < k_hi) ? d : -INFINITY;
+      s[j] = (key >= t_lo && key < t_hi) ? d - slope * (float)(pos - key) : -INFINITY;
       tmax = fmaxf(tmax, s[j]);
     }
     tmax = wave_max(tmax);
@@ -301,13 +327,13 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
           Mj = M2;
         }
       }
-      put((T*)p.out + out_at(p, row, h * HD + tid), aj / Lj);
+      put((T*)p.out + out_at(p, row, h * HD + tid), aj / Lj * gate_at<T>(p, row, h * HD + tid));
     }
     return;
   }
   if (tid < HD) {
     if (n_splits == 1) {
-      put((T*)p.out + out_at(p, row, h * HD + tid), acc / L);
+      put((T*)p.out + out_at(p, row, h * HD + tid), acc / L * gate_at<T>(p, row, h * HD + tid));
     } else {
       const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
       p.part_o[base * HD + tid] = acc;
@@ -333,7 +359,7 @@ __global__ void attn_decode_merge_kernel(DecodeArgs p) {
     L += p.part_ml[(base + s) * 2 + 1] * w;
     acc += p.part_o[(base + s) * HD + d] * w;
   }
-  put((T*)p.out + out_at(p, row, h * HD + d), acc / L);
+  put((T*)p.out + out_at(p, row, h * HD + d), acc / L * gate_at<T>(p, row, h * HD + d));
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
@@ -365,15 +391,19 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
 // 65,536 (row, head)s; part_o and part_ml are still where the parts pass through); 2, the same,
 // and n_splits is only the most a row takes: a short row takes fewer, by its own length.
 // Launches that join in the kernel and overlap on one GPU race (they share the counters).
-extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                                const void* v_pages, size_t page_stride, const int* block_table,
-                                int max_blocks, const int* token_req, const int* positions,
-                                const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                                int page_size, int window, float scale, int n_splits, float* part_o,
-                                float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                                int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
-                                int join_in_kernel, hipStream_t stream) {
+// attn_decode_rows_biased: with the optional terms of DecodeArgs (null or 0 where one is absent).
+extern "C" int attn_decode_rows_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                       const void* v_pages, size_t page_stride, const int* block_table,
+                                       int max_blocks, const int* token_req, const int* positions,
+                                       const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                       int page_size, int window, float scale, int n_splits, float* part_o,
+                                       float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                       int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                                       int join_in_kernel, const float* head_scale, const float* slopes,
+                                       const void* gate, int ldg, int keep_first, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (keep_first < 0) FAIL("attn_decode: keep_first %d must not be negative", keep_first);
+  if (gate && ldg < n_heads * head_dim) FAIL("attn_decode: the gate's row stride %d is smaller than its rows", ldg);
   if (key_tile == 0) key_tile = 32;
   if (key_tile != 32 && key_tile != 64) FAIL("attn_decode: a wave takes 32 or 64 keys at a time, not %d", key_tile);
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("attn_decode: unknown dtype code %d", dtype);
@@ -405,6 +435,8 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
   p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size;
   p.window = window, p.n_splits = n_splits, p.scale = scale;
+  p.head_scale = head_scale, p.slopes = slopes, p.gate = gate, p.ldg = ldg;
+  p.keep_first = window > 0 ? keep_first : 0;
   if (ahead && (((uintptr_t)ahead & 15) || ahead_chunk_bytes % 16 != 0 || ahead_chunks < 0))
     FAIL("attn_decode: what is read ahead must be chunks of 16-byte pieces");
   p.ahead = (const uint4*)ahead, p.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
@@ -433,4 +465,19 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
   }
   CHECK_LAUNCH("attn_decode");
   return 0;
+}
+
+extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                const void* v_pages, size_t page_stride, const int* block_table,
+                                int max_blocks, const int* token_req, const int* positions,
+                                const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                int page_size, int window, float scale, int n_splits, float* part_o,
+                                float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                                int join_in_kernel, hipStream_t stream) {
+  return attn_decode_rows_biased(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                                 positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                                 n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks,
+                                 rows_are_requests, dtype, key_tile, join_in_kernel, nullptr, nullptr, nullptr, 0, 0,
+                                 stream);
 }

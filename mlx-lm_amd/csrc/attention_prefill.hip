@@ -40,6 +40,14 @@ struct PrefillArgs {
   int n_heads, n_kv_heads, page_size, window;
   int page_shift;  // log2(page_size), or -1 if that is no power of two
   float scale;
+  // Optional terms (the kernel's EXTRAS variant; all absent: plain causal attention), as in
+  // attention.hip's AttnArgs: head_scale [n_heads] instead of `scale`; slopes [n_heads], slope *
+  // distance taken off a score; keep_first, the first keys that a window leaves visible; gate
+  // (bfloat16 rows of stride ldg), the output times its sigmoid.
+  const float* head_scale;
+  const float* slopes;
+  const uint16_t* gate;
+  int ldg, keep_first;
 };
 
 #define BQ ATTN_PREFILL_TILE_QUERIES  // queries per block
@@ -58,7 +66,8 @@ __device__ __forceinline__ int key_of_row(int rho) {
 }
 
 // POW2: the page size is a power of two (a key's page and row are a shift and a mask)
-template <int HD, bool POW2>
+// EXTRAS: the optional terms of PrefillArgs are looked at (the plain variant has no trace of them)
+template <int HD, bool POW2, bool EXTRAS>
 __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(PrefillArgs p) {
   constexpr int KS_STRIDE = HD + 8;
   constexpr int DC = HD / 16;           // 16-column chunks of a head (QK contraction steps)
@@ -107,7 +116,12 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   // keys this wave's queries can see end here; later tiles it only helps to load
   const int wave_hi = min(k_hi, pos0 + wave * 32 + 32);
   const int wave_q0 = pos0 + wave * 32;            // position of the wave's first query
-  const float c2 = p.scale * 1.4426950408889634f;  // scores to units of log 2
+  const float c2 = (EXTRAS && p.head_scale ? p.head_scale[h] : p.scale) * 1.4426950408889634f;  // scores to units of log 2
+  const float slope2 = EXTRAS && p.slopes ? p.slopes[h] * 1.4426950408889634f : 0.f;
+  // the kept first keys [0, sink_hi) that the tile's window has left behind: tiles of their own, first
+  const int sink_hi = EXTRAS ? min(p.window > 0 ? p.keep_first : 0, k_lo) : 0;
+  const int n_sink_tiles = (sink_hi + KT - 1) / KT;
+  const int n_sink_pages = sink_hi > 0 ? (sink_hi - 1) / p.page_size + 1 : 0;
 
   float m = -INFINITY, l = 0.f;
   f32x16_t ot[DT];
@@ -127,7 +141,8 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   extern __shared__ int page_of[];  // [max_blocks]
   const int pg0 = k_lo / p.page_size;
   const int n_pg = (k_hi - 1) / p.page_size - pg0 + 1;
-  for (int i = tid; i < n_pg; i += 256) page_of[i] = table[pg0 + i];
+  for (int i = tid; i < n_sink_pages; i += 256) page_of[i] = table[i];
+  for (int i = tid; i < n_pg; i += 256) page_of[n_sink_pages + i] = table[pg0 + i];
   __syncthreads();
 
   // Loads are never predicated and never zeroed: a key outside [k_lo, k_hi) is
@@ -139,8 +154,12 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   // choice is the kernel's template argument, and everything but the page's start is 32-bit.
   const uint32_t stride32 = (uint32_t)p.page_stride;
   const int shift = p.page_shift, row_mask = p.page_size - 1;
+  // (a tile's first key says of which run it is: at or beyond 2^29, the kept first keys')
+  constexpr int SINK = 1 << 29;
   auto address = [&](int key, int col) __attribute__((always_inline)) -> size_t {
-    const int kk = min(max(key, k_lo), k_hi - 1);
+    int kk = min(max(key, k_lo), k_hi - 1);
+    int first_page = pg0 - n_sink_pages;
+    if (EXTRAS && key >= SINK) kk = min(key - SINK, sink_hi - 1), first_page = 0;
     int idx, row;
     if constexpr (POW2) {
       idx = kk >> shift, row = kk & row_mask;
@@ -148,7 +167,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
       idx = kk / p.page_size, row = kk - idx * p.page_size;
     }
     const uint32_t within = head_off + (uint32_t)(row * HD + col);
-    return (size_t)(uint32_t)page_of[idx - pg0] * stride32 + within;
+    return (size_t)(uint32_t)page_of[idx - first_page] * stride32 + within;
   };
   auto fetch = [&](int kt, const int set) __attribute__((always_inline)) {
 #pragma unroll
@@ -196,14 +215,17 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   // and there is no window, so no wave is idle and nothing is masked; a loop of
   // such tiles has no branch inside, and the compiler lets the loads of the
   // other register set stay in flight while this one is staged.
-  auto one_tile = [&](int kt, const int set, auto steady) __attribute__((always_inline)) {
+  // `kt_next2`: the first key of the tile after the next (its loads start here).
+  auto one_tile = [&](int kt_in, int kt_next2, const int set, auto steady) __attribute__((always_inline)) {
     constexpr bool STEADY = decltype(steady)::value;
     __syncthreads();  // the previous tile is no longer read
     stage(set);
     __syncthreads();
-    fetch(kt + 2 * KT, set);  // (beyond the last tile: harmless reads of the last key)
+    fetch(kt_next2, set);  // (beyond the last tile: harmless reads of the last key)
+    const bool sink = EXTRAS && kt_in >= SINK;
+    const int kt = sink ? kt_in - SINK : kt_in;
     if constexpr (!STEADY) {
-      if (kt >= wave_hi || wave * 32 >= nq) return;  // nothing here for this wave (uniform)
+      if ((!sink && kt >= wave_hi) || wave * 32 >= nq) return;  // nothing here for this wave (uniform)
     }
 
     // ---- S^T = K Q^T for the two 32-key subtiles --------------------------------
@@ -226,9 +248,23 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
     // v_exp_f32.  Tiles that every query of the wave sees whole (below the
     // diagonal, inside the window) skip the masks: this arithmetic, not the
     // MFMAs, is what the kernel's time goes to.
-    const bool whole = STEADY || (kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
+    const bool whole = STEADY || (!EXTRAS && kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
     float tmax = -INFINITY;
-    if (whole) {
+    if constexpr (EXTRAS) {
+      // scores in units of log 2 with the distance's share taken off; a key counts if it is of
+      // this tile's run and the query sees it (inside its window, or one of the kept first)
+      const int run_lo = sink ? 0 : k_lo, run_hi = sink ? sink_hi : k_hi;
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kt + 32 * s + 16 * (r >> 3) + 8 * g + (r & 7);
+          const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
+          const float v = fmaf(st[s][r], c2, -slope2 * (float)(qpos - key));
+          st[s][r] = ok ? v : -INFINITY;
+          tmax = fmaxf(tmax, st[s][r]);
+        }
+    } else if (whole) {
 #pragma unroll
       for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -258,7 +294,8 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
         float e[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          e[i] = __builtin_amdgcn_exp2f(fmaf(st[s][8 * c + i], c2, -m_use));
+          e[i] = EXTRAS ? __builtin_amdgcn_exp2f(st[s][8 * c + i] - m_use)
+                        : __builtin_amdgcn_exp2f(fmaf(st[s][8 * c + i], c2, -m_use));
           lsum += e[i];
         }
         pf[s][c].u.x = pack_bf16x2(e[0], e[1]);
@@ -288,19 +325,33 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
     }
   };
 
-  fetch(kt0, 0);
-  fetch(kt0 + KT, 1);
-  int kt = kt0;
-  if (p.window <= 0) {
-    for (; kt + 2 * KT - 1 <= pos0; kt += 2 * KT) {
-      one_tile(kt, 0, std::true_type{});
-      one_tile(kt + KT, 1, std::true_type{});
+  if constexpr (EXTRAS) {
+    // tile i of the walk: the kept first keys' tiles, then the window's (beyond the last: the
+    // window's go on, whose loads are harmless reads of the last key)
+    auto first_key = [&](int i) { return i < n_sink_tiles ? SINK + i * KT : kt0 + (i - n_sink_tiles) * KT; };
+    const int n_all = n_sink_tiles + (k_hi - kt0 + KT - 1) / KT;
+    fetch(first_key(0), 0);
+    fetch(first_key(1), 1);
+    for (int i = 0; i < n_all; i += 2) {
+      one_tile(first_key(i), first_key(i + 2), 0, std::false_type{});
+      if (i + 1 >= n_all) break;  // uniform
+      one_tile(first_key(i + 1), first_key(i + 3), 1, std::false_type{});
     }
-  }
-  for (; kt < k_hi; kt += 2 * KT) {  // the tiles around the diagonal, or all of them under a window
-    one_tile(kt, 0, std::false_type{});
-    if (kt + KT >= k_hi) break;  // uniform
-    one_tile(kt + KT, 1, std::false_type{});
+  } else {
+    fetch(kt0, 0);
+    fetch(kt0 + KT, 1);
+    int kt = kt0;
+    if (p.window <= 0) {
+      for (; kt + 2 * KT - 1 <= pos0; kt += 2 * KT) {
+        one_tile(kt, kt + 2 * KT, 0, std::true_type{});
+        one_tile(kt + KT, kt + 3 * KT, 1, std::true_type{});
+      }
+    }
+    for (; kt < k_hi; kt += 2 * KT) {  // the tiles around the diagonal, or all of them under a window
+      one_tile(kt, kt + 2 * KT, 0, std::false_type{});
+      if (kt + KT >= k_hi) break;  // uniform
+      one_tile(kt + KT, kt + 3 * KT, 1, std::false_type{});
+    }
   }
 
   // the two halves of the wave hold different keys of the same query
@@ -313,9 +364,17 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // accumulators 4j .. 4j+3: head columns dt*32 + 8j + 4g + (0..3)
+        float w[4] = {inv, inv, inv, inv};
+        if (EXTRAS && p.gate) {
+          const uint2 gv = *(const uint2*)(p.gate + (size_t)(row0 + qi) * p.ldg + h * HD + dt * 32 + 8 * j + 4 * g);
+          const float gf[4] = {__uint_as_float(gv.x << 16), __uint_as_float(gv.x & 0xffff0000u),
+                               __uint_as_float(gv.y << 16), __uint_as_float(gv.y & 0xffff0000u)};
+#pragma unroll
+          for (int c = 0; c < 4; ++c) w[c] = inv / (1.0f + expf(-gf[c]));
+        }
         uint2 o;
-        o.x = pack_bf16x2(ot[dt][4 * j] * inv, ot[dt][4 * j + 1] * inv);
-        o.y = pack_bf16x2(ot[dt][4 * j + 2] * inv, ot[dt][4 * j + 3] * inv);
+        o.x = pack_bf16x2(ot[dt][4 * j] * w[0], ot[dt][4 * j + 1] * w[1]);
+        o.y = pack_bf16x2(ot[dt][4 * j + 2] * w[2], ot[dt][4 * j + 3] * w[3]);
         *(uint2*)(orow + dt * 32 + 8 * j + 4 * g) = o;
       }
   }
@@ -326,13 +385,18 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 // tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
 // bfloat16 only, head_dim 32, 64 or 128.
-extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                            const void* v_pages, size_t page_stride, const int* block_table,
-                            int max_blocks, const int* token_req, const int* positions,
-                            const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
-                            int head_dim, int page_size, int window, float scale,
-                            hipStream_t stream) {
+// attn_prefill_biased: with the optional terms of PrefillArgs (null or 0 where one is absent).
+extern "C" int attn_prefill_biased(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                   const void* v_pages, size_t page_stride, const int* block_table,
+                                   int max_blocks, const int* token_req, const int* positions,
+                                   const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                                   int head_dim, int page_size, int window, float scale,
+                                   const float* head_scale, const float* slopes, const void* gate, int ldg,
+                                   int keep_first, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (keep_first < 0) FAIL("attn_prefill: keep_first %d must not be negative", keep_first);
+  if (gate && (ldg < n_heads * head_dim || ldg % 4 != 0 || ((uintptr_t)gate & 7)))
+    FAIL("attn_prefill: the gate's rows (stride %d) must be 8-byte aligned and as wide as the output's", ldg);
   if (head_dim != 32 && head_dim != 64 && head_dim != 128)
     FAIL("attn_prefill: head_dim %d is not 32, 64 or 128 (attn_tile takes the others)", head_dim);
   if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
@@ -356,16 +420,23 @@ extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const vo
     if ((1 << sh) == page_size) p.page_shift = sh;
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size, p.window = window;
   p.scale = scale;
+  p.head_scale = head_scale, p.slopes = slopes, p.gate = (const uint16_t*)gate, p.ldg = ldg;
+  p.keep_first = window > 0 ? keep_first : 0;
+  const bool extras = head_scale || slopes || gate || p.keep_first > 0;
   if (n_tiles > 65535) FAIL("attn_prefill: %d tiles in a launch, at most 65535", n_tiles);
   dim3 grid(n_heads, n_tiles), block(256);
   // a request's page numbers lie in LDS beside the tiles
   if (max_blocks > 7168)
     FAIL("attn_prefill: block tables of %d pages a request do not fit beside the tiles (at most 7168)", max_blocks);
-  const size_t lds = (size_t)max_blocks * sizeof(int);
+  // (the kept first keys' pages lie before the window's; a page can be in both runs)
+  const size_t lds = (size_t)(max_blocks + (extras ? 2 : 0)) * sizeof(int);
   const bool pow2 = p.page_shift >= 0;
-#define LAUNCH_PREFILL(HD)                                                                    \
-  if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true>), grid, block, lds, stream, p); \
-  else hipLaunchKernelGGL((attn_prefill_kernel<HD, false>), grid, block, lds, stream, p)
+#define LAUNCH_PREFILL(HD)                                                                                  \
+  if (extras) {                                                                                             \
+    if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true, true>), grid, block, lds, stream, p);      \
+    else hipLaunchKernelGGL((attn_prefill_kernel<HD, false, true>), grid, block, lds, stream, p);          \
+  } else if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true, false>), grid, block, lds, stream, p); \
+  else hipLaunchKernelGGL((attn_prefill_kernel<HD, false, false>), grid, block, lds, stream, p)
   if (head_dim == 32) {
     LAUNCH_PREFILL(32);
   } else if (head_dim == 64) {
@@ -376,4 +447,15 @@ extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const vo
 #undef LAUNCH_PREFILL
   CHECK_LAUNCH("attn_prefill");
   return 0;
+}
+
+extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                            const void* v_pages, size_t page_stride, const int* block_table,
+                            int max_blocks, const int* token_req, const int* positions,
+                            const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                            int head_dim, int page_size, int window, float scale,
+                            hipStream_t stream) {
+  return attn_prefill_biased(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                             positions, tiles, n_tiles, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                             nullptr, nullptr, nullptr, 0, 0, stream);
 }

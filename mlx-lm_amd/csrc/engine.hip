@@ -49,8 +49,8 @@ extern "C" int eng_compute_units(void) { return n_compute_units(); }
 
 // The decode kernel's waves a block where rows are few, and the keys a wave from which a row's keys
 // are split over blocks (the kernel narrows a launch's splits row by row with the same number).
-#define ROW_WAVES 8
-#define ROW_SPLIT_KEYS_A_WAVE 96
+#define ROW_WAVES ATTN_DECODE_ROW_WAVES
+#define ROW_SPLIT_KEYS_A_WAVE ATTN_DECODE_SPLIT_KEYS_A_WAVE
 
 // The context length from which a decode step may split a row's keys over blocks (what a recorded
 // step's planning length is chosen by: below it no step launches splits).
@@ -705,28 +705,7 @@ struct Attention : Mixer {
   void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves,
                 int* key_tile) const {
     const long c = window <= 0 ? max_row_context : (max_row_context < window + 31 ? max_row_context : window + 31);
-    const long tiles = c + 31 < 32 ? 1 : (c + 31) / 32;
-    const long blocks = n_rows * n_heads < 1 ? 1 : (long)n_rows * n_heads;
-    int nw = blocks > ctx->n_compute_units ? 4 : ROW_WAVES;
-    const int fewest = head_dim > 128 ? 4 : 2;  // (the block's threads write a column of the head each)
-    while (nw > fewest && nw / 2 >= tiles) nw /= 2;
-    const long keys_a_wave = c / nw;
-    long ns = 1;
-    if (keys_a_wave >= ROW_SPLIT_KEYS_A_WAVE) {
-      ns = keys_a_wave / 32;
-      if (ctx->n_compute_units / blocks < ns) ns = ctx->n_compute_units / blocks;
-      if (ns > 64) ns = 64;
-      if (ns < 1) ns = 1;
-    }
-    *n_splits = (int)ns, *n_waves = nw, *key_tile = 32;
-    if (blocks > 3 * ctx->n_compute_units && c >= 640) {
-      // many rows and a long walk: tiles of 64 keys, and as many waves a block as make eight a CU
-      // (32 rows: four; 64 rows: two.  With four at 64 rows the step took 5.92 ms instead of 5.76.)
-      const long want = (8L * ctx->n_compute_units + blocks - 1) / blocks;
-      nw = fewest;
-      while (nw < 8 && nw < want) nw *= 2;
-      *n_waves = nw, *key_tile = 64;
-    }
+    attn_decode_row_work(ctx->n_compute_units, n_rows, n_heads, head_dim, c, n_splits, n_waves, key_tile);
   }
 
   // How many ways to split a row's keys so that the general row kernel's launch fills the GPU.

@@ -86,7 +86,15 @@ typedef int (*fn_attn_tile_biased)(void*, const void*, int, int, const void*, co
 typedef int (*fn_attn_row_biased)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                                   const int*, const int*, const int*, int, int, int, int, int, int, float, int, float*,
                                   float*, int, const float*, const float*, const void*, int, int, hipStream_t);
+typedef int (*fn_attn_prefill_biased)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                      const int*, const int*, const int*, int, int, int, int, int, int, float,
+                                      const float*, const float*, const void*, int, int, hipStream_t);
+typedef int (*fn_attn_decode_biased)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
+                                     const int*, const int*, const int*, int, int, int, int, int, int, float, int,
+                                     float*, float*, int, const void*, size_t, int, int, int, int, int, const float*,
+                                     const float*, const void*, int, int, hipStream_t);
 typedef const char* (*fn_error)();
+#define ROW_KERNEL_MAX_HEAD_DIM 144  // beyond it the tile kernel takes single rows too
 
 // the attention part's step arrays, from `array_base` on (parts/attention.py)
 enum { ARR_TILES = 0, ARR_ROWS, ARR_ALL_TILES, ARR_BIG_TILES, ARR_MAX_ROW_CONTEXT, ARR_ROWS_ARE_REQUESTS };
@@ -100,7 +108,9 @@ struct GatedKeyAttention : Mixer {
   const float* slopes;      // [n_heads]
   fn_attn_tile_biased attn_tile = nullptr;
   fn_attn_row_biased attn_row = nullptr;
-  fn_error attn_error = nullptr;
+  fn_attn_prefill_biased attn_prefill = nullptr;
+  fn_attn_decode_biased attn_decode = nullptr;
+  fn_error attn_error = nullptr, prefill_error = nullptr, decode_error = nullptr;
 
   GatedKeyAttention() { can_overwrite = true; }
 
@@ -113,6 +123,24 @@ struct GatedKeyAttention : Mixer {
         attn_tile = nullptr;
         return host->fail("gated key attention: the 'attention' kernels are not loaded");
       }
+    }
+    return 0;
+  }
+  // (the kernels for the head sizes that the matrix cores and the register-streaming rows take
+  // are in libraries of their own, looked up only where a model has such heads)
+  int prefill_kernel() {
+    if (!attn_prefill) {
+      attn_prefill = (fn_attn_prefill_biased)host->kernel("attention_prefill", "attn_prefill_biased");
+      prefill_error = (fn_error)host->kernel("attention_prefill", "mlxlm_last_error");
+      if (!attn_prefill || !prefill_error) return host->fail("gated key attention: the 'attention_prefill' kernels are not loaded");
+    }
+    return 0;
+  }
+  int decode_kernel() {
+    if (!attn_decode) {
+      attn_decode = (fn_attn_decode_biased)host->kernel("attention_decode", "attn_decode_rows_biased");
+      decode_error = (fn_error)host->kernel("attention_decode", "mlxlm_last_error");
+      if (!attn_decode || !decode_error) return host->fail("gated key attention: the 'attention_decode' kernels are not loaded");
     }
     return 0;
   }
@@ -156,32 +184,74 @@ struct GatedKeyAttention : Mixer {
     const char* gate = (const char*)qkg.p + (size_t)(q_width + kv_width) * (ctx->dtype == DT_BF16 ? 2 : 4);
     const int* tiles = ctx->arrays[array_base + ARR_TILES];
     const int* rows = ctx->arrays[array_base + ARR_ROWS];
+    const int* all_tiles = ctx->arrays[array_base + ARR_ALL_TILES];
+    const int* big_tiles = ctx->arrays[array_base + ARR_BIG_TILES];
     const int n_tiles = (int)ctx->counts[array_base + ARR_TILES] / 2;
     const int n_rows = (int)ctx->counts[array_base + ARR_ROWS];
+    const int n_all_tiles = (int)ctx->counts[array_base + ARR_ALL_TILES] / 2;
+    const int n_big_tiles = (int)ctx->counts[array_base + ARR_BIG_TILES] / 2;
     const long longest = ctx->counts[array_base + ARR_MAX_ROW_CONTEXT];
+    const int rows_are_requests = ctx->counts[array_base + ARR_ROWS_ARE_REQUESTS] != 0;
     if (n_tiles == 0 && n_rows == 0) return host->fail("gated key attention: the step carries no work lists for its %d rows", T);
-    if (n_tiles) {
+    const bool bf16 = ctx->dtype == DT_BF16;
+    // which kernel takes which rows: as the plain attention part chooses (tiles of 128 queries on
+    // the matrix cores for bfloat16 heads of 32, 64 or 128; single rows through registers where a
+    // key is 64, 128 or 256 bytes; the general tile and row kernels otherwise)
+    if (head_dim > ROW_KERNEL_MAX_HEAD_DIM) {
       if (attn_tile(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks, kv.token_req,
-                    kv.positions, tiles, n_tiles, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f, ctx->dtype,
-                    head_scale, slopes, gate, qkg.ld, keep_first, ctx->stream))
+                    kv.positions, all_tiles, n_all_tiles, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f,
+                    ctx->dtype, head_scale, slopes, gate, qkg.ld, keep_first, ctx->stream))
         return host->fail("%s", attn_error());
       host->launched(ctx);
-    }
-    if (n_rows) {
-      const int n_splits = row_splits(ctx, n_rows, longest);
-      if (ctx->stats && n_splits > ctx->stats->key_splits_most) ctx->stats->key_splits_most = n_splits;
-      EngMat part_o = {}, part_ml = {};
-      if (n_splits > 1) {
-        const long n = (long)n_rows * n_heads * n_splits;
-        if (host->take(ctx, 1, (int)(n * head_dim), DT_F32, &part_o)) return 1;
-        if (host->take(ctx, 1, (int)(n * 2), DT_F32, &part_ml)) return 1;
+    } else {
+      if (n_tiles && bf16 && (head_dim == 32 || head_dim == 64 || head_dim == 128)) {
+        if (prefill_kernel()) return 1;
+        if (attn_prefill(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks,
+                         kv.token_req, kv.positions, big_tiles, n_big_tiles, n_heads, n_kv_heads, head_dim, kv.page_size,
+                         window, 1.f, head_scale, slopes, gate, qkg.ld, keep_first, ctx->stream))
+          return host->fail("%s", prefill_error());
+        host->launched(ctx);
+      } else if (n_tiles) {
+        if (attn_tile(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks, kv.token_req,
+                      kv.positions, tiles, n_tiles, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f, ctx->dtype,
+                      head_scale, slopes, gate, qkg.ld, keep_first, ctx->stream))
+          return host->fail("%s", attn_error());
+        host->launched(ctx);
       }
-      if (attn_row(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks, kv.token_req,
-                   kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f, n_splits,
-                   (float*)part_o.p, (float*)part_ml.p, ctx->dtype, head_scale, slopes, gate, qkg.ld, keep_first,
-                   ctx->stream))
-        return host->fail("%s", attn_error());
-      host->launched(ctx);
+      if (n_rows) {
+        const int key_bytes = head_dim * (bf16 ? 2 : 4);
+        const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) && kv.page_size % (1024 / key_bytes) == 0;
+        int n_splits = 1, n_waves = 4, key_tile = 32;
+        if (fast) {
+          long keys = longest;
+          if (window > 0 && keys > window + keep_first + 62) keys = window + keep_first + 62;
+          attn_decode_row_work(ctx->n_compute_units, n_rows, n_heads, head_dim, keys, &n_splits, &n_waves, &key_tile);
+        } else {
+          n_splits = row_splits(ctx, n_rows, longest);
+        }
+        if (ctx->stats && n_splits > ctx->stats->key_splits_most) ctx->stats->key_splits_most = n_splits;
+        EngMat part_o = {}, part_ml = {};
+        if (n_splits > 1) {
+          const long n = (long)n_rows * n_heads * n_splits;
+          if (host->take(ctx, 1, (int)(n * head_dim), DT_F32, &part_o)) return 1;
+          if (host->take(ctx, 1, (int)(n * 2), DT_F32, &part_ml)) return 1;
+        }
+        if (fast) {
+          if (decode_kernel()) return 1;
+          if (attn_decode(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks, kv.token_req,
+                          kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f, n_splits,
+                          (float*)part_o.p, (float*)part_ml.p, n_waves, nullptr, 0, 0, rows_are_requests, ctx->dtype,
+                          key_tile, 2, head_scale, slopes, gate, qkg.ld, keep_first, ctx->stream))
+            return host->fail("%s", decode_error());
+        } else {
+          if (attn_row(o.p, qkg.p, qkg.ld, o.ld, kv.k, kv.v, kv.page_stride, kv.block_table, kv.max_blocks, kv.token_req,
+                       kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim, kv.page_size, window, 1.f, n_splits,
+                       (float*)part_o.p, (float*)part_ml.p, ctx->dtype, head_scale, slopes, gate, qkg.ld, keep_first,
+                       ctx->stream))
+            return host->fail("%s", attn_error());
+        }
+        host->launched(ctx);
+      }
     }
     EngLinear out = {};
     out.out = y, out.a.m = o, out.w = out_w, out.accumulate = overwrite ? 0 : 1;

@@ -556,10 +556,37 @@ def kv_write(k_src, v_src, kv, block_table, token_req, positions):
     build.check(lib, rc, "kv_write")
 
 
-def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0):
+class ScoreTerms:
+    """Optional terms that the four attention kernels take beside the plain causal scores:
+    ``head_scale`` (float32 ``[n_heads]``, instead of ``scale``), ``slopes`` (float32 ``[n_heads]``:
+    ``slope * (query position - key position)`` is taken off a score), ``gate`` (``[tokens,
+    n_heads * head_dim]`` of the queries' dtype: the output is multiplied by its sigmoid) and
+    ``keep_first`` (with a window, the first so many keys stay visible)."""
+
+    def __init__(self, head_scale=None, slopes=None, gate=None, keep_first=0):
+        self.head_scale, self.slopes, self.gate, self.keep_first = head_scale, slopes, gate, int(keep_first)
+
+    def args(self, q, n_heads):
+        for name in ("head_scale", "slopes"):
+            t = getattr(self, name)
+            if t is not None:
+                _dev(t, name, torch.float32)
+                _need(t.numel() == n_heads, f"{name}: one value a head")
+        ldg = 0
+        if self.gate is not None:
+            ldg = _rows2d(self.gate, "gate")
+            _need(self.gate.dtype == q.dtype and self.gate.shape == q.shape, "gate: the queries' shape and dtype")
+        return [_ptr(self.head_scale), _ptr(self.slopes), _ptr(self.gate), _c_int(ldg), _c_int(self.keep_first)]
+
+
+def _terms(terms, q, n_heads):
+    return (terms or ScoreTerms()).args(q, n_heads)
+
+
+def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0, terms=None):
     """Attention for tiles of up to 16 consecutive queries of one request each.
 
-    ``tiles`` is int32 ``[n_tiles, 2]``: first flat row and number of rows.
+    ``tiles`` is int32 ``[n_tiles, 2]``: first flat row and number of rows.  ``terms``: ``ScoreTerms``.
     """
     lib = build.load("attention")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
@@ -568,12 +595,12 @@ def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_h
     _attn_common(q, kv, block_table, token_req, positions)
     _dev(tiles, "tiles", torch.int32)
     _need(tiles.numel() >= 2 * n_tiles, "attn_tile: tile list too short")
-    rc = lib.attn_tile(
+    rc = lib.attn_tile_biased(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
-        _c_float(scale), _c_int(DT[q.dtype]), _stream(),
+        _c_float(scale), _c_int(DT[q.dtype]), *_terms(terms, q, n_heads), _stream(),
     )
     build.check(lib, rc, "attn_tile")
     return out
@@ -583,7 +610,7 @@ ATTN_ROW_MAX_HEAD_DIM = 144  # beyond this the per-wave key tiles do not fit in 
 
 
 def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
-             window=0, n_splits=1, part_o=None, part_ml=None):
+             window=0, n_splits=1, part_o=None, part_ml=None, terms=None):
     """Attention for single query rows, keys split ``n_splits`` ways."""
     lib = build.load("attention")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
@@ -599,13 +626,13 @@ def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_head
         _dev(part_ml, "part_ml", torch.float32)
         _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_row: part_o too small")
         _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_row: part_ml too small")
-    rc = lib.attn_row(
+    rc = lib.attn_row_biased(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
         _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(DT[q.dtype]),
-        _stream(),
+        *_terms(terms, q, n_heads), _stream(),
     )
     build.check(lib, rc, "attn_row")
     return out
@@ -637,7 +664,7 @@ def attn_prefill_takes(q_dtype, kv):
     return q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)
 
 
-def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0):
+def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0, terms=None):
     """``attn_tile`` on the matrix cores: bfloat16, head_dim 32/64/128, tiles of up to 128 queries."""
     lib = build.load("attention_prefill")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
@@ -647,12 +674,12 @@ def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, 
     _attn_common(q, kv, block_table, token_req, positions)
     _dev(tiles, "tiles", torch.int32)
     _need(tiles.numel() >= 2 * n_tiles, "attn_prefill: tile list too short")
-    rc = lib.attn_prefill(
+    rc = lib.attn_prefill_biased(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
-        _c_float(scale), _stream(),
+        _c_float(scale), *_terms(terms, q, n_heads), _stream(),
     )
     build.check(lib, rc, "attn_prefill")
     return out
@@ -668,7 +695,7 @@ def attn_decode_takes(q_dtype, kv):
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
                 window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0,
-                rows_are_requests=False, key_tile=32, join_in_kernel=0):
+                rows_are_requests=False, key_tile=32, join_in_kernel=0, terms=None):
     """``attn_row`` for keys of 64, 128 or 256 bytes (bfloat16 with head_dim 32, 64 or 128, float32
     with 16, 32 or 64): keys stream into registers.
 
@@ -696,7 +723,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_decode: part_ml too small")
     if rows_are_requests:
         _need(n_rows <= block_table.shape[0], "attn_decode: more rows than requests")
-    rc = lib.attn_decode_rows(
+    rc = lib.attn_decode_rows_biased(
         _ptr(out.data if packed_out else out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
@@ -706,7 +733,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
         _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0),
         _c_int(1 if rows_are_requests else 0), _c_int(DT[q.dtype]), _c_int(key_tile),
-        _c_int(int(join_in_kernel)), _stream(),
+        _c_int(int(join_in_kernel)), *_terms(terms, q, n_heads), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

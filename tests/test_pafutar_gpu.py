@@ -13,7 +13,7 @@ import pytest
 import torch
 
 import helpers
-import plain_pafutar as plain
+import plain_pafutar as plain  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -284,7 +284,7 @@ def test_windows_give_pages_back_and_stale_pages_do_not_matter(models, page_size
 
     eng.add_request("r")
     rows, i = [], 0
-    for c in [30, 2, 17] + [1] * 60 + [9, 20, 11] + [1] * 100:
+    for c in [30, 2, 17] + [1] * 60 + [9, 20, 11] + [1] * 101:
         rows.append(eng.step([StepEntry("r", tokens[i : i + c], list(range(c)))]).clone())
         i += c
         eng.cache.poison_free_pages()
@@ -400,3 +400,89 @@ def test_trace_replay_of_a_random_model(tmp_path, models):
     want = plain.forward(weights, config, tokens)
     got = np.fromfile(out / "1.f32", dtype="<f4").reshape(-1, config["vocab"])
     _close(torch.from_numpy(got), want[31:], "float32", "the replay's second step")
+
+
+# -- the attention kernels with the optional score terms, each against the plain formulas ------
+
+
+def _paged(keys, values, page_size, dtype, seed):
+    """Keys and values ``[n, G, d]`` in pages handed out in a shuffled order; the rest holds NaN."""
+    from mlx_lm_amd.ops.kernels import PagedKV
+
+    n, G, d = keys.shape
+    n_blocks = (n + page_size - 1) // page_size
+    order = torch.randperm(n_blocks + 3, generator=torch.Generator().manual_seed(seed))[:n_blocks]
+    both = torch.full((n_blocks + 3, 2, G, page_size, d), float("nan"), dtype=dtype, device="cuda")
+    for b in range(n_blocks):
+        rows = slice(b * page_size, min(n, (b + 1) * page_size))
+        m = rows.stop - rows.start
+        both[order[b], 0, :, :m] = keys[rows].permute(1, 0, 2).to(dtype)
+        both[order[b], 1, :, :m] = values[rows].permute(1, 0, 2).to(dtype)
+        both[order[b], :, :, m:] = 0  # (rows of a page that are not written yet hold numbers)
+    return PagedKV(both[:, 0], both[:, 1]), order.to(torch.int32).cuda()[None].contiguous()
+
+
+@pytest.mark.parametrize("kernel,dtype,d", [("tile", torch.float32, 48), ("tile", torch.bfloat16, 24), ("row", torch.float32, 40),
+                                            ("row", torch.bfloat16, 96), ("prefill", torch.bfloat16, 64),
+                                            ("prefill", torch.bfloat16, 128), ("prefill", torch.bfloat16, 32),
+                                            ("decode", torch.bfloat16, 64), ("decode", torch.float32, 64),
+                                            ("decode", torch.bfloat16, 128)])
+@pytest.mark.parametrize("window,keep_first", [(0, 0), (50, 0), (50, 7), (37, 70), (300, 21)])
+def test_attention_kernels_with_score_terms(kernel, dtype, d, window, keep_first):
+    """Queries at positions 530 .. of a request that holds 530 + n keys: temperatures, distance
+    slopes, a window with kept first keys (more of them than a page or a tile, or fewer than the
+    window leaves behind) and the gate, against softmax((q.k) c_h - m_h (i - j)) v * sigmoid(g)."""
+    from mlx_lm_amd.ops import kernels
+
+    H, G, offset = 4, 2, 530
+    n_q = {"tile": 16, "row": 3, "prefill": 150, "decode": 3}[kernel]
+    n = offset + n_q
+    g = torch.Generator().manual_seed(d + window + keep_first)
+    q = torch.randn(n_q, H, d, generator=g).to(dtype)
+    k = torch.randn(n, G, d, generator=g).to(dtype)
+    v = torch.randn(n, G, d, generator=g).to(dtype)
+    gate = torch.randn(n_q, H * d, generator=g).to(dtype)
+    temp = torch.rand(H, generator=g) * 2.0 / d**0.5 + 0.5 / d**0.5  # scores with a spread of a few units
+    # Keys that stand out for the first query's last head (the one with the gentlest slope): the
+    # last kept key and the one after it, the key just inside the window and the one just outside.
+    # Taken for the wrong side of its edge, any of them moves the output by about its value.
+    if window:
+        edges = [(offset - window, 1.2), (offset - window + 1, 1.2)]
+        edges += [(keep_first - 1, 1.8), (keep_first, 1.8)] if keep_first else []  # (far away: the slope takes more off)
+        for j, factor in edges:
+            if 0 <= j < n:
+                k[j, G - 1] = (q[0, H - 1].float() * factor).to(dtype)
+    slopes = plain.head_slopes(H).float()
+    # the plain side: scores with scale 1 and the heads' temperatures, the mask, the gate
+    s = plain.attention_scores(q.double(), k.double(), 1.0, temp.double(), offset)
+    see = plain.visible(n_q, offset, window if window else n + 1, keep_first)[:, :n]
+    p = torch.softmax(s.masked_fill(~see.unsqueeze(0), float("-inf")), dim=-1)
+    want = torch.einsum("hij,jhd->ihd", p, v.double().repeat_interleave(H // G, dim=1)).reshape(n_q, H * d)
+    want = want * torch.sigmoid(gate.double())
+    if window and keep_first:
+        assert p[H - 1, 0, keep_first - 1] > 0.1  # the first query leans on the last kept key
+
+    kv, table = _paged(k, v, 16, dtype, seed=d)
+    qd = q.reshape(n_q, H * d).cuda()
+    out = torch.empty_like(qd)
+    zeros = torch.zeros(n_q, dtype=torch.int32, device="cuda")
+    positions = (torch.arange(n_q, dtype=torch.int32) + offset).cuda()
+    terms = kernels.ScoreTerms(temp.cuda(), slopes.cuda(), gate.cuda(), keep_first)
+    rows = torch.arange(n_q, dtype=torch.int32).cuda()
+    if kernel == "tile":
+        tiles = torch.tensor([[0, n_q]], dtype=torch.int32).cuda()
+        kernels.attn_tile(out, qd, kv, table, zeros, positions, tiles, 1, H, 1.0, window, terms)
+    elif kernel == "prefill":
+        tiles = torch.tensor([[128, n_q - 128], [0, 128]], dtype=torch.int32).cuda()
+        kernels.attn_prefill(out, qd, kv, table, zeros, positions, tiles, 2, H, 1.0, window, terms)
+    else:
+        n_splits = 3
+        part_o = torch.empty(n_q * H * n_splits * d, device="cuda")
+        part_ml = torch.empty(n_q * H * n_splits * 2, device="cuda")
+        if kernel == "row":
+            kernels.attn_row(out, qd, kv, table, zeros, positions, rows, n_q, H, 1.0, window, n_splits, part_o, part_ml, terms)
+        else:
+            kernels.attn_decode(out, qd, kv, table, zeros, positions, rows, n_q, H, 1.0, window, n_splits, part_o, part_ml,
+                                n_waves=4, join_in_kernel=2, terms=terms)
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err <= (2e-5 if dtype == torch.float32 else 2.5e-2) * want.abs().max().item(), err
