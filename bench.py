@@ -25,6 +25,14 @@ the host's clock around an evaluated result).  Weights are random (seeded), data
 positions and, unless ``--layers`` says otherwise, 12 of the 48 layers (``config`` names both);
 ``value`` is decode at batch 8 from context 7,000, ``points`` hold batch 1 and 8 at contexts 4,000
 and 7,000, ``prefill`` is one prompt of 8,192 tokens.
+
+``--designs`` is another mode of its own (the default workload and its line are untouched by it):
+Pafutar beside GPT-2 at equal sizes (the same width, heads, head size, inner size, layers,
+vocabulary and positions; every Pafutar head with a key head of its own, as GPT-2's), random weights,
+prefill of 2 x 1,024 tokens and decode at batch 1, 8 and 32 from context 512, for each of
+``DESIGN_SIZES`` (``--design-size`` names one, ``--design-only`` one design, for a profile).  The
+Pafutar model runs once without a window (like for like with GPT-2's attention) and once with a
+window of 512 that keeps the first 64 tokens.  It prints one JSON line of its own.
 """
 
 import argparse
@@ -43,6 +51,85 @@ PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
 XL = dict(model_type="gpt2", n_layer=48, n_embd=1600, n_head=25, n_inner=6400, vocab_size=50257,
           n_positions=1024, n_ctx=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+
+
+# Layer sizes for --designs: width = heads x head size, as GPT-2 has it
+DESIGN_SIZES = {
+    "1024": dict(width=1024, heads=16, dim=64, ff=4096, layers=12),
+    "2048": dict(width=2048, heads=16, dim=128, ff=8192, layers=8),
+}
+DESIGN_VOCAB, DESIGN_POSITIONS = 32000, 2048
+
+
+def design_config(design, size, window=None):
+    """The config.json of ``design`` ("gpt2", "pafutar") at one of ``DESIGN_SIZES``."""
+    s = DESIGN_SIZES[size]
+    if design == "gpt2":
+        return dict(model_type="gpt2", n_layer=s["layers"], n_embd=s["width"], n_head=s["heads"], n_inner=s["ff"],
+                    vocab_size=DESIGN_VOCAB, n_positions=DESIGN_POSITIONS, layer_norm_epsilon=1e-5,
+                    activation_function="gelu_new")
+    mixer = {"heads": s["heads"], "kv_heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5}
+    if window:
+        mixer["mask"] = {"size": window[0], "keep_first": window[1]}
+    layer = {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": s["ff"]}}
+    return {"architecture": "Pafutar", "vocab": DESIGN_VOCAB, "width": s["width"], "max_positions": DESIGN_POSITIONS,
+            "embedding": {"scale": s["width"] ** 0.5}, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
+            "layers": [dict(layer) for _ in range(s["layers"])]}
+
+
+def bench_design(config, dtype, batches, steps, warmup):
+    """Prefill of 2 x 1,024 tokens (three warm-up trials, the mean of five) and decode from
+    context 512 at each of ``batches``, for the model that ``config`` describes."""
+    import torch
+
+    from mlx_lm_amd.engine import Engine, StepEntry
+
+    model, _ = build_model(config, dtype, seed=2)
+    V, P = model.decoder.vocab_size, model.decoder.max_positions
+    engine = Engine(model, dtype=dtype, page_size=16, max_tokens=max(batches) * 1024 + 4096, max_requests=64,
+                    record_prompt_steps=True)
+    g = torch.Generator().manual_seed(0)
+    prompts = torch.randint(0, V, (2, 1024), generator=g).tolist()
+    ms = []
+    for trial in range(8):
+        for i in range(2):
+            engine.add_request(("pre", i))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry(("pre", i), prompts[i], [1023]) for i in range(2)])
+        torch.cuda.synchronize()
+        ms.append((time.perf_counter() - t0) * 1e3)
+        for i in range(2):
+            engine.end_request(("pre", i))
+    pre = sum(ms[3:]) / 5
+    out = {"prefill_ms": round(pre, 3), "prefill_tok_s": round(2048 / (pre / 1e3), 1),
+           "weight_bytes": model.decoder.bytes_read_per_step(2 if dtype == "bfloat16" else 4)}
+    for b in batches:
+        dt, contexts = run_decode(engine, b, 512, min(steps, P - 514), warmup, V, seed=b)
+        k = len(contexts)
+        step_bytes = out["weight_bytes"] + b * (sum(contexts) / k) * engine.cache.bytes_per_token()
+        out[f"decode_b{b}"] = {"tok_s": round(b * k / dt, 1), "ms_per_step": round(dt / k * 1e3, 4),
+                               "hbm_frac": round(step_bytes / (dt / k) / 1e9 / PEAK_HBM_GBS, 4)}
+    print(f"[bench] {config.get('model_type') or config.get('architecture')}: {out}", file=sys.stderr, flush=True)
+    return out
+
+
+def compare_designs(a):
+    """The ``--designs`` mode: one JSON line with both designs' numbers at every size."""
+    sizes = [a.design_size] if a.design_size else list(DESIGN_SIZES)
+    batches = [1, 8, 32]
+    line = {"metric": "prefill tok/s (2 x 1,024) and decode tok/s from context 512: Pafutar beside GPT-2 at equal sizes",
+            "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic token ids, random weights (seed 2)",
+            "steps": a.steps, "warmup": a.warmup, "vocab": DESIGN_VOCAB, "positions": DESIGN_POSITIONS, "sizes": {}}
+    for size in sizes:
+        entry = {"layer_sizes": DESIGN_SIZES[size]}
+        runs = {"gpt2": ("gpt2", None), "pafutar": ("pafutar", None), "pafutar_window_512_keep_64": ("pafutar", (512, 64))}
+        for name, (design, window) in runs.items():
+            if a.design_only and name != a.design_only:
+                continue
+            entry[name] = bench_design(design_config(design, size, window), a.dtype, batches, a.steps, a.warmup)
+        line["sizes"][size] = entry
+    print(json.dumps(line))
 
 
 def build_model(config, dtype, seed):
@@ -142,7 +229,17 @@ def main():
     ap.add_argument("--n-positions", type=int, default=XL["n_positions"],
                     help="positions of the model; 8192: the long-context mode (12 layers unless --layers is given)")
     ap.add_argument("--no-points", action="store_true", help="skip the other batch sizes and contexts")
+    ap.add_argument("--designs", action="store_true",
+                    help="a mode of its own: Pafutar beside GPT-2 at equal layer sizes (prefill and decode)")
+    ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default=None, help="with --designs: one size only")
+    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64")
     a = ap.parse_args()
+    if a.designs:
+        if a.gpus != 1:
+            print("bench.py measures one GPU; this engine does not run on several (asked for %d)" % a.gpus)
+            sys.exit(2)
+        a.steps = min(a.steps, 128)
+        return compare_designs(a)
     long_mode = a.n_positions != XL["n_positions"]
     if a.layers is None:
         a.layers = 12 if long_mode else XL["n_layer"]

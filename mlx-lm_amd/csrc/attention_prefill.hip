@@ -251,19 +251,40 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
     const bool whole = STEADY || (!EXTRAS && kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
     float tmax = -INFINITY;
     if constexpr (EXTRAS) {
-      // scores in units of log 2 with the distance's share taken off; a key counts if it is of
-      // this tile's run and the query sees it (inside its window, or one of the kept first)
-      const int run_lo = sink ? 0 : k_lo, run_hi = sink ? sink_hi : k_hi;
+      // Scores in units of log 2 with the distance's share taken off: element r of subtile s is
+      // the key kt + 8 g + off(s, r) with off a constant of the element, so the share is
+      // slope2 * (off - (qpos - kt - 8 g)), one multiply-add on top of the score's own.
+      const float far = slope2 * (float)(qpos - kt - 8 * g);
+      // A tile that every query of the wave sees whole (below the diagonal and inside the window,
+      // or all of it kept first keys) needs no masks.
+      const bool all_seen = sink ? kt + KT <= sink_hi
+                                 : (kt >= k_lo && kt + KT - 1 <= wave_q0 && wave_q0 + 31 < nq + pos0 &&
+                                    (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
+      if (all_seen) {
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kt + 32 * s + 16 * (r >> 3) + 8 * g + (r & 7);
-          const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
-          const float v = fmaf(st[s][r], c2, -slope2 * (float)(qpos - key));
-          st[s][r] = ok ? v : -INFINITY;
-          tmax = fmaxf(tmax, st[s][r]);
-        }
+          for (int r = 0; r < 16; ++r) {
+            const float off = (float)(32 * s + 16 * (r >> 3) + (r & 7));
+            st[s][r] = fmaf(st[s][r], c2, fmaf(slope2, off, -far));
+            tmax = fmaxf(tmax, st[s][r]);
+          }
+      } else {
+        // a key counts if it is of this tile's run and the query sees it (inside its window, or
+        // one of the kept first)
+        const int run_lo = sink ? 0 : k_lo, run_hi = sink ? sink_hi : k_hi;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int o = 32 * s + 16 * (r >> 3) + (r & 7);
+            const int key = kt + 8 * g + o;
+            const bool ok = q_live && key <= qpos && key >= run_lo && key < run_hi && (key >= q_lo || key < p.keep_first);
+            const float v = fmaf(st[s][r], c2, fmaf(slope2, (float)o, -far));
+            st[s][r] = ok ? v : -INFINITY;
+            tmax = fmaxf(tmax, st[s][r]);
+          }
+      }
     } else if (whole) {
 #pragma unroll
       for (int s = 0; s < 2; ++s)

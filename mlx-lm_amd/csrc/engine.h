@@ -55,7 +55,7 @@ typedef struct {
   int rows, cols, ld, n_splits;
   float* ws;
   const float* bias;
-  int allowed, pad_;
+  int allowed, pad_;  // allowed: 0 no; 1 a sum into the stream may stay pending; 2 also a product that writes float32 rows
 } EngPending;
 
 // One cache slot: pages of keys and values, or a state tensor, or nothing.  A slot of per-request

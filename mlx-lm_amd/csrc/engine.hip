@@ -324,7 +324,10 @@ extern "C" int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, i
 // the second kernel adds the parts and runs the epilogue.
 static int finish_parts(EngCtx* ctx, const EngMat& out, float* ws, int n_splits, const float* bias, int gelu,
                         bool accumulate, const EngScatter* sc, EngPending* pending, bool out_packed = false) {
-  if (accumulate && pending && pending->allowed) {
+  // (allowed == 2: whoever reads `out` next adds the parts up itself, also where the product
+  // writes its float32 rows instead of adding to them; `out` itself is not touched then)
+  const bool writes_plain = !accumulate && !gelu && !sc && !out_packed && out.dtype == DT_F32 && out.ld == out.cols;
+  if (pending && ((accumulate && pending->allowed) || (writes_plain && pending->allowed == 2))) {
     pending->target = (float*)out.p, pending->rows = out.rows, pending->cols = out.cols, pending->ld = out.ld;
     pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
     return 0;

@@ -13,7 +13,9 @@
 #include "engine_parts.h"
 #include "attention_tiles.h"
 
-// grid (n_tokens), 256 threads: a wave takes the heads w, w + 4, ... (the query heads, then the key heads)
+// grid (n_tokens, ceil((n_heads + n_kv_heads) / 4)), 256 threads: a wave a head (the query heads,
+// then the key heads), its columns in registers (up to four a lane: head sizes to 256), so that a
+// head costs one trip to memory
 template <typename T>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(T* __restrict__ qk, int ld, int n_heads, int n_kv_heads,
                                                          int head_dim, float eps, T* __restrict__ k_pages,
@@ -21,30 +23,32 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(T* __restrict__ qk, int
                                                          const int* __restrict__ block_table, int max_blocks,
                                                          const int* __restrict__ token_req,
                                                          const int* __restrict__ positions, int page_size) {
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  T* row = qk + (size_t)t * ld;
-  size_t page_at = 0;
-  if (k_pages) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const int u = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (u >= n_heads + n_kv_heads) return;  // (whole waves; no barrier follows)
+  T* v = qk + (size_t)t * ld + (size_t)u * head_dim;  // (the keys' columns follow the queries')
+  T raw[4];
+  float f[4], q = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    raw[i] = v[min(d, head_dim - 1)];
+    f[i] = d < head_dim ? to_f32(raw[i]) : 0.f;
+    q += f[i] * f[i];
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)head_dim + eps);
+  if (u < n_heads) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (lane + 64 * i < head_dim) v[lane + 64 * i] = from_f32<T>(f[i] * rstd);
+  } else if (k_pages) {
     const int pos = positions[t];
     const int page = block_table[(size_t)token_req[t] * max_blocks + pos / page_size];
-    page_at = (size_t)page * page_stride + (size_t)(pos % page_size) * head_dim;
-  }
-  for (int u = wave; u < n_heads + n_kv_heads; u += 4) {
-    T* v = row + (size_t)u * head_dim;  // (the keys' columns follow the queries')
-    float q = 0.f;
-    for (int d = lane; d < head_dim; d += 64) {
-      const float f = to_f32(v[d]);
-      q += f * f;
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)head_dim + eps);
-    if (u < n_heads) {
-      for (int d = lane; d < head_dim; d += 64) v[d] = from_f32<T>(to_f32(v[d]) * rstd);
-    } else if (k_pages) {
-      const size_t dst = page_at + (size_t)(u - n_heads) * page_size * head_dim;
-      for (int d = lane; d < head_dim; d += 64) {
-        v_pages[dst + d] = v[d];
-        k_pages[dst + d] = from_f32<T>(to_f32(v[d]) * rstd);
-      }
+    const size_t dst = (size_t)page * page_stride + ((size_t)(u - n_heads) * page_size + pos % page_size) * head_dim;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < head_dim) v_pages[dst + d] = raw[i], k_pages[dst + d] = from_f32<T>(f[i] * rstd);
     }
   }
 }
@@ -57,12 +61,12 @@ extern "C" int qk_prepare(void* qk, int ld, int n_tokens, int n_heads, int n_kv_
                           void* k_pages, void* v_pages, size_t page_stride, const int* block_table, int max_blocks,
                           const int* token_req, const int* positions, int page_size, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
-  if (!qk || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || ld < (n_heads + n_kv_heads) * head_dim)
+  if (!qk || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || head_dim > 256 || ld < (n_heads + n_kv_heads) * head_dim)
     FAIL("qk_prepare: %d + %d heads of %d in rows of stride %d", n_heads, n_kv_heads, head_dim, ld);
   if (k_pages && (!v_pages || !block_table || !token_req || !positions || page_size <= 0 ||
                   page_stride < (size_t)n_kv_heads * page_size * head_dim))
     FAIL("qk_prepare: the cache write needs pages, block table, token_req and positions");
-  dim3 grid(n_tokens), block(256);
+  dim3 grid(n_tokens, (n_heads + n_kv_heads + 3) / 4), block(256);
   if (dtype == DT_F32)
     hipLaunchKernelGGL(qk_prepare_kernel<float>, grid, block, 0, stream, (float*)qk, ld, n_heads, n_kv_heads, head_dim, eps,
                        (float*)k_pages, (float*)v_pages, page_stride, block_table, max_blocks, token_req, positions, page_size);
@@ -173,7 +177,7 @@ struct GatedKeyAttention : Mixer {
     if (host->take(ctx, T, 2 * q_width + kv_width, ctx->dtype, &qkg)) return 1;
     EngLinear call = {};
     call.out = qkg, call.a = x, call.w = qkg_w, call.bias = qkg_b;
-    if (host->linear(ctx, &call, &ctx->pending)) return 1;
+    if (host->linear(ctx, &call, nullptr)) return 1;  // (nothing of this product may stay pending)
     if (qk_prepare(qkg.p, qkg.ld, T, n_heads, n_kv_heads, head_dim, eps, writes ? kv.k : nullptr, kv.v, kv.page_stride,
                    kv.block_table, kv.max_blocks, kv.token_req, kv.positions, kv.page_size, ctx->dtype, ctx->stream))
       return host->fail("%s", g_err);

@@ -16,12 +16,115 @@
 #include "common.h"
 #include "engine_parts.h"
 
-template <typename T>
+// A block a row, the row in registers (NV float4 a thread, width <= 1024 NV): every load of the
+// row is on its way before the first is used, so a row costs one trip to memory, not one a
+// stretch of 64 columns.  Columns beyond the width are read from inside it and dropped.
+template <typename T, int NV>
 __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out, const float* __restrict__ x, int ldx,
                                                           const float* __restrict__ mu,
                                                           const float* __restrict__ state, size_t state_stride,
                                                           const int* __restrict__ slot_ids,
-                                                          const int* __restrict__ token_req, int n_rows, int width) {
+                                                          const int* __restrict__ token_req, int width) {
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* xr = x + (size_t)r * ldx;
+  const float* prev = xr;
+  if (mu) {
+    const int req = token_req[r];
+    const bool first = r == 0 || token_req[r - 1] != req;  // a request's rows are consecutive
+    prev = first ? state + (size_t)slot_ids[req] * state_stride : xr - ldx;
+  }
+  float4 v[NV], pv[NV], m[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = min((tid + 256 * i) * 4, width - 4);
+    v[i] = *(const float4*)(xr + k);
+    if (mu) pv[i] = *(const float4*)(prev + k), m[i] = *(const float4*)(mu + k);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    if (k >= width) continue;
+    float o[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+    if (mu) {
+      o[0] += (pv[i].x - v[i].x) * m[i].x, o[1] += (pv[i].y - v[i].y) * m[i].y;
+      o[2] += (pv[i].z - v[i].z) * m[i].z, o[3] += (pv[i].w - v[i].w) * m[i].w;
+    }
+    T* at = out + (size_t)r * width + k;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) at[c] = from_f32<T>(o[c]);
+  }
+}
+
+// y: the sublayer's output rows (null: nothing but the parts); parts: n_parts partial products
+// [n_parts][n_rows][width] that still have to be added up (a product that split its inner size).
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void residual_rmsnorm_kernel(float* __restrict__ h, int ldh,
+                                                               const float* __restrict__ y, int ldy,
+                                                               const float* __restrict__ parts, int n_parts,
+                                                               float alpha, const float* __restrict__ s,
+                                                               const float* __restrict__ gamma, float eps,
+                                                               float* __restrict__ state, size_t state_stride,
+                                                               const int* __restrict__ slot_ids,
+                                                               const int* __restrict__ token_req,
+                                                               T* __restrict__ copy, int n_rows, int width) {
+  __shared__ float red[32];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  float* hr = h + (size_t)r * ldh;
+  float* keep = nullptr;
+  if (state) {
+    const int req = token_req[r];
+    if (r == n_rows - 1 || token_req[r + 1] != req) keep = state + (size_t)slot_ids[req] * state_stride;
+  }
+  float4 old[NV], out[NV], sc[NV], g[NV];
+  const size_t part_step = (size_t)n_rows * width;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = min((tid + 256 * i) * 4, width - 4);
+    old[i] = *(const float4*)(hr + k);
+    out[i] = y ? *(const float4*)(y + (size_t)r * ldy + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    sc[i] = s ? *(const float4*)(s + k) : make_float4(1.f, 1.f, 1.f, 1.f);
+    g[i] = gamma ? *(const float4*)(gamma + k) : make_float4(1.f, 1.f, 1.f, 1.f);
+    const float* pr = parts + (size_t)r * width + k;
+    for (int p0 = 0; p0 < n_parts; p0 += 4) {  // four parts' loads at a time, added in their order
+      float4 t[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t[j] = *(const float4*)(pr + min(p0 + j, n_parts - 1) * part_step);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (p0 + j < n_parts) out[i].x += t[j].x, out[i].y += t[j].y, out[i].z += t[j].z, out[i].w += t[j].w;
+    }
+  }
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    out[i].x = alpha * old[i].x + sc[i].x * out[i].x, out[i].y = alpha * old[i].y + sc[i].y * out[i].y;
+    out[i].z = alpha * old[i].z + sc[i].z * out[i].z, out[i].w = alpha * old[i].w + sc[i].w * out[i].w;
+    if (k < width) q += (out[i].x * out[i].x + out[i].y * out[i].y) + (out[i].z * out[i].z + out[i].w * out[i].w);
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    if (k >= width) continue;
+    if (keep) *(float4*)(keep + k) = old[i];
+    const float4 n = make_float4(out[i].x * rstd * g[i].x, out[i].y * rstd * g[i].y, out[i].z * rstd * g[i].z,
+                                 out[i].w * rstd * g[i].w);
+    *(float4*)(hr + k) = n;
+    if (copy) {
+      T* at = copy + (size_t)r * width + k;
+      at[0] = from_f32<T>(n.x), at[1] = from_f32<T>(n.y), at[2] = from_f32<T>(n.z), at[3] = from_f32<T>(n.w);
+    }
+  }
+}
+
+// The same two for any width and alignment: a wave a row, a column a lane at a time.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_any_kernel(T* __restrict__ out, const float* __restrict__ x, int ldx,
+                                                              const float* __restrict__ mu,
+                                                              const float* __restrict__ state, size_t state_stride,
+                                                              const int* __restrict__ slot_ids,
+                                                              const int* __restrict__ token_req, int n_rows, int width) {
   const int lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;
@@ -32,7 +135,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out, c
     return;
   }
   const int req = token_req[r];
-  const bool first = r == 0 || token_req[r - 1] != req;  // a request's rows are consecutive
+  const bool first = r == 0 || token_req[r - 1] != req;
   const float* prev = first ? state + (size_t)slot_ids[req] * state_stride : xr - ldx;
   for (int k = lane; k < width; k += 64) {
     const float v = xr[k];
@@ -41,35 +144,39 @@ __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out, c
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void residual_rmsnorm_kernel(float* __restrict__ h, int ldh,
-                                                               const float* __restrict__ y, int ldy, float alpha,
-                                                               const float* __restrict__ s,
-                                                               const float* __restrict__ gamma, float eps,
-                                                               float* __restrict__ state, size_t state_stride,
-                                                               const int* __restrict__ slot_ids,
-                                                               const int* __restrict__ token_req,
-                                                               T* __restrict__ copy, int n_rows, int width) {
+__global__ __launch_bounds__(256) void residual_rmsnorm_any_kernel(float* __restrict__ h, int ldh,
+                                                                   const float* __restrict__ y, int ldy,
+                                                                   const float* __restrict__ parts, int n_parts,
+                                                                   float alpha, const float* __restrict__ s,
+                                                                   const float* __restrict__ gamma, float eps,
+                                                                   float* __restrict__ state, size_t state_stride,
+                                                                   const int* __restrict__ slot_ids,
+                                                                   const int* __restrict__ token_req,
+                                                                   T* __restrict__ copy, int n_rows, int width) {
   const int lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;
   float* hr = h + (size_t)r * ldh;
-  const float* yr = y + (size_t)r * ldy;
   float* keep = nullptr;
   if (state) {
     const int req = token_req[r];
     if (r == n_rows - 1 || token_req[r + 1] != req) keep = state + (size_t)slot_ids[req] * state_stride;
   }
+  const size_t part_step = (size_t)n_rows * width;
+  auto sum_at = [&](int k) {
+    float v = y ? y[(size_t)r * ldy + k] : 0.f;
+    for (int p = 0; p < n_parts; ++p) v += parts[p * part_step + (size_t)r * width + k];
+    return alpha * hr[k] + (s ? s[k] : 1.f) * v;
+  };
   float q = 0.f;
   for (int k = lane; k < width; k += 64) {
-    const float old = hr[k];
-    if (keep) keep[k] = old;
-    const float v = alpha * old + (s ? s[k] : 1.f) * yr[k];
+    if (keep) keep[k] = hr[k];
+    const float v = sum_at(k);
     q += v * v;
   }
   const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
   for (int k = lane; k < width; k += 64) {
-    const float v = alpha * hr[k] + (s ? s[k] : 1.f) * yr[k];
-    const float n = v * rstd * (gamma ? gamma[k] : 1.f);
+    const float n = sum_at(k) * rstd * (gamma ? gamma[k] : 1.f);
     hr[k] = n;
     if (copy) copy[(size_t)r * width + k] = from_f32<T>(n);
   }
@@ -82,6 +189,22 @@ __global__ void zero_rows_kernel(float* p, size_t n) {
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// NV float4 a thread cover `width` columns with 256 threads; 0: too wide for the registers
+static inline int vectors_for(int width) {
+  const int nv = (width / 4 + 255) / 256;
+  return nv <= 1 ? 1 : nv <= 2 ? 2 : nv <= 4 ? 4 : nv <= 8 ? 8 : 0;
+}
+
+#define BY_VECTORS(nv, LAUNCH) \
+  do {                         \
+    if (nv == 1) LAUNCH(1);    \
+    else if (nv == 2) LAUNCH(2); \
+    else if (nv == 4) LAUNCH(4); \
+    else LAUNCH(8);            \
+  } while (0)
+
 // out [n_rows, width] (out_dtype) = shift(x); mu null: a conversion.  state [slots, state_stride] float32.
 extern "C" int token_shift(void* out, const float* x, int ldx, const float* mu, const float* state,
                            size_t state_stride, const int* slot_ids, const int* token_req, int n_rows, int width,
@@ -91,40 +214,75 @@ extern "C" int token_shift(void* out, const float* x, int ldx, const float* mu, 
   if (!out || !x) FAIL("token_shift: null pointer");
   if (mu && (!state || !slot_ids || !token_req || state_stride < (size_t)width))
     FAIL("token_shift: the shift needs the state tensor (rows of %d), slot ids and token_req", width);
-  dim3 grid((n_rows + 3) / 4), block(256);
-  if (out_dtype == DT_F32)
-    hipLaunchKernelGGL(token_shift_kernel<float>, grid, block, 0, stream, (float*)out, x, ldx, mu, state, state_stride,
-                       slot_ids, token_req, n_rows, width);
-  else if (out_dtype == DT_BF16)
-    hipLaunchKernelGGL(token_shift_kernel<bf16>, grid, block, 0, stream, (bf16*)out, x, ldx, mu, state, state_stride,
-                       slot_ids, token_req, n_rows, width);
-  else
-    FAIL("token_shift: unknown dtype code %d", out_dtype);
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("token_shift: unknown dtype code %d", out_dtype);
+  const int nv = vectors_for(width);
+  const bool vec = nv > 0 && width % 4 == 0 && ldx % 4 == 0 && state_stride % 4 == 0 && aligned16(x) && aligned16(mu) &&
+                   aligned16(state);
+  if (vec) {
+#define LAUNCH(NV)                                                                                                     \
+  if (out_dtype == DT_F32)                                                                                             \
+    hipLaunchKernelGGL((token_shift_kernel<float, NV>), dim3(n_rows), dim3(256), 0, stream, (float*)out, x, ldx, mu,  \
+                       state, state_stride, slot_ids, token_req, width);                                              \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((token_shift_kernel<bf16, NV>), dim3(n_rows), dim3(256), 0, stream, (bf16*)out, x, ldx, mu,    \
+                       state, state_stride, slot_ids, token_req, width)
+    BY_VECTORS(nv, LAUNCH);
+#undef LAUNCH
+  } else {
+    dim3 grid((n_rows + 3) / 4), block(256);
+    if (out_dtype == DT_F32)
+      hipLaunchKernelGGL(token_shift_any_kernel<float>, grid, block, 0, stream, (float*)out, x, ldx, mu, state,
+                         state_stride, slot_ids, token_req, n_rows, width);
+    else
+      hipLaunchKernelGGL(token_shift_any_kernel<bf16>, grid, block, 0, stream, (bf16*)out, x, ldx, mu, state,
+                         state_stride, slot_ids, token_req, n_rows, width);
+  }
   CHECK_LAUNCH("token_shift");
   return 0;
 }
 
-// h [n_rows, width] float32 (row stride ldh) <- N(alpha h + s * y) * gamma, in place.  s, gamma: null = ones.
-// state non-null: the old row that ends each request's run of rows goes to the request's row of it.
-// copy non-null: the new rows once more, contiguous, in copy_dtype.
-extern "C" int residual_rmsnorm(float* h, int ldh, const float* y, int ldy, float alpha, const float* s,
-                                const float* gamma, float eps, float* state, size_t state_stride,
-                                const int* slot_ids, const int* token_req, void* copy, int copy_dtype, int n_rows,
-                                int width, hipStream_t stream) {
+// h [n_rows, width] float32 (row stride ldh) <- N(alpha h + s * (y + the parts)) * gamma, in place.
+// y: the sublayer's rows (null: none); parts: n_parts partial products [n_parts][n_rows][width] still
+// to be added (null: none).  s, gamma: null = ones.  state non-null: the old row that ends each
+// request's run of rows goes to the request's row of it.  copy non-null: the new rows once more,
+// contiguous, in copy_dtype.
+extern "C" int residual_rmsnorm(float* h, int ldh, const float* y, int ldy, const float* parts, int n_parts,
+                                float alpha, const float* s, const float* gamma, float eps, float* state,
+                                size_t state_stride, const int* slot_ids, const int* token_req, void* copy,
+                                int copy_dtype, int n_rows, int width, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (width <= 0 || ldh < width || ldy < width) FAIL("residual_rmsnorm: width %d, row strides %d and %d", width, ldh, ldy);
-  if (!h || !y) FAIL("residual_rmsnorm: null pointer");
+  if (width <= 0 || ldh < width || (y && ldy < width)) FAIL("residual_rmsnorm: width %d, row strides %d and %d", width, ldh, ldy);
+  if (!h || (!y && !parts)) FAIL("residual_rmsnorm: null pointer");
+  if (!parts) n_parts = 0;
+  if (n_parts < 0) FAIL("residual_rmsnorm: %d parts", n_parts);
   if (state && (!slot_ids || !token_req || state_stride < (size_t)width))
     FAIL("residual_rmsnorm: keeping rows needs slot ids, token_req and state rows of %d", width);
-  dim3 grid((n_rows + 3) / 4), block(256);
-  if (copy && copy_dtype == DT_BF16)
-    hipLaunchKernelGGL(residual_rmsnorm_kernel<bf16>, grid, block, 0, stream, h, ldh, y, ldy, alpha, s, gamma, eps, state,
-                       state_stride, slot_ids, token_req, (bf16*)copy, n_rows, width);
-  else if (!copy || copy_dtype == DT_F32)
-    hipLaunchKernelGGL(residual_rmsnorm_kernel<float>, grid, block, 0, stream, h, ldh, y, ldy, alpha, s, gamma, eps, state,
-                       state_stride, slot_ids, token_req, (float*)copy, n_rows, width);
-  else
-    FAIL("residual_rmsnorm: unknown dtype code %d", copy_dtype);
+  if (copy && copy_dtype != DT_F32 && copy_dtype != DT_BF16) FAIL("residual_rmsnorm: unknown dtype code %d", copy_dtype);
+  const bool half = copy && copy_dtype == DT_BF16;
+  const int nv = vectors_for(width);
+  const bool vec = nv > 0 && width % 4 == 0 && ldh % 4 == 0 && ldy % 4 == 0 && state_stride % 4 == 0 && aligned16(h) &&
+                   aligned16(y) && aligned16(parts) && aligned16(s) && aligned16(gamma) && aligned16(state);
+  if (vec) {
+#define LAUNCH(NV)                                                                                                       \
+  if (half)                                                                                                              \
+    hipLaunchKernelGGL((residual_rmsnorm_kernel<bf16, NV>), dim3(n_rows), dim3(256), 0, stream, h, ldh, y, ldy, parts,   \
+                       n_parts, alpha, s, gamma, eps, state, state_stride, slot_ids, token_req, (bf16*)copy, n_rows,    \
+                       width);                                                                                          \
+  else                                                                                                                   \
+    hipLaunchKernelGGL((residual_rmsnorm_kernel<float, NV>), dim3(n_rows), dim3(256), 0, stream, h, ldh, y, ldy, parts,  \
+                       n_parts, alpha, s, gamma, eps, state, state_stride, slot_ids, token_req, (float*)copy, n_rows,   \
+                       width)
+    BY_VECTORS(nv, LAUNCH);
+#undef LAUNCH
+  } else {
+    dim3 grid((n_rows + 3) / 4), block(256);
+    if (half)
+      hipLaunchKernelGGL(residual_rmsnorm_any_kernel<bf16>, grid, block, 0, stream, h, ldh, y, ldy, parts, n_parts, alpha,
+                         s, gamma, eps, state, state_stride, slot_ids, token_req, (bf16*)copy, n_rows, width);
+    else
+      hipLaunchKernelGGL(residual_rmsnorm_any_kernel<float>, grid, block, 0, stream, h, ldh, y, ldy, parts, n_parts, alpha,
+                         s, gamma, eps, state, state_stride, slot_ids, token_req, (float*)copy, n_rows, width);
+  }
   CHECK_LAUNCH("residual_rmsnorm");
   return 0;
 }
@@ -144,6 +302,24 @@ struct PostNormBlock : Block {
   const float* scale1 = nullptr;  // null: the sublayer's output as it is
   const float* scale2 = nullptr;
   const float* mu = nullptr;  // null: no shift
+
+  // What the sum-and-norm reads for a sublayer's output: its rows, or (and) parts still pending on them.
+  struct Parts {
+    const float* y;
+    const float* ws;
+    int n;
+  };
+  int take_parts(EngCtx* ctx, const EngMat& y, bool y_holds_rows, Parts* out) {
+    EngPending* p = &ctx->pending;
+    out->y = (const float*)y.p, out->ws = nullptr, out->n = 0;
+    if (!p->target) return 0;
+    if ((void*)p->target != y.p || p->rows != y.rows || p->cols != y.cols || p->ld != y.cols || p->bias)
+      return host->settle(ctx, p);  // (a sum of another shape: added the plain way)
+    out->ws = p->ws, out->n = p->n_splits;
+    if (!y_holds_rows) out->y = nullptr;  // (a product that writes left nothing but its parts)
+    p->target = nullptr;
+    return 0;
+  }
 
   int zero(EngCtx* ctx, const EngMat& y) {
     const size_t n = (size_t)y.rows * y.ld;
@@ -180,8 +356,17 @@ struct PostNormBlock : Block {
     }
     EngMat y;
     if (host->take(ctx, T, width, DT_F32, &y)) return 1;
+    // A sublayer's last product may split its inner size and leave the parts where they are
+    // (EngPending.allowed == 2: also a product that writes, not adds): the sum-and-norm adds them up.
+    EngPending* pending = &ctx->pending;
+    if (host->settle(ctx, pending)) return 1;
+    pending->allowed = 2;
     if (!mixer->overwrite && zero(ctx, y)) return 1;
-    if (int rc = mixer->forward(ctx, u, y, slot, writes)) return rc;
+    int rc = mixer->forward(ctx, u, y, slot, writes);
+    pending->allowed = 0;
+    if (rc) return rc;
+    Parts parts;
+    if (take_parts(ctx, y, !mixer->overwrite, &parts)) return 1;
     // the first sum and norm; the rows that end a portion are kept for the next step's shift; the
     // feed-forward's product reads a copy in the compute dtype
     EngValue x = {};
@@ -189,15 +374,20 @@ struct PostNormBlock : Block {
     if (ffn && ctx->dtype != DT_F32) {
       if (host->take(ctx, T, width, ctx->dtype, &x.m)) return 1;
     }
-    if (residual_rmsnorm((float*)h.p, h.ld, (const float*)y.p, y.ld, alpha, scale1, gamma1, eps, state, state_stride,
-                         ctx->slot_ids, ctx->token_req, x.m.p != h.p ? x.m.p : nullptr, ctx->dtype, T, width, ctx->stream))
+    if (residual_rmsnorm((float*)h.p, h.ld, parts.y, y.ld, parts.ws, parts.n, alpha, scale1, gamma1, eps, state,
+                         state_stride, ctx->slot_ids, ctx->token_req, x.m.p != h.p ? x.m.p : nullptr, ctx->dtype, T, width,
+                         ctx->stream))
       return host->fail("%s", g_err);
     host->launched(ctx);
     if (ffn) {
+      pending->allowed = 2;
       if (!ffn->overwrite && zero(ctx, y)) return 1;
-      if (int rc = ffn->forward(ctx, x, y)) return rc;
-      if (residual_rmsnorm((float*)h.p, h.ld, (const float*)y.p, y.ld, alpha, scale2, gamma2, eps, nullptr, 0, nullptr,
-                           nullptr, nullptr, 0, T, width, ctx->stream))
+      rc = ffn->forward(ctx, x, y);
+      pending->allowed = 0;
+      if (rc) return rc;
+      if (take_parts(ctx, y, !ffn->overwrite, &parts)) return 1;
+      if (residual_rmsnorm((float*)h.p, h.ld, parts.y, y.ld, parts.ws, parts.n, alpha, scale2, gamma2, eps, nullptr, 0,
+                           nullptr, nullptr, nullptr, 0, T, width, ctx->stream))
         return host->fail("%s", g_err);
       host->launched(ctx);
     }

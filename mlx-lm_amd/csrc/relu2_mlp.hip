@@ -18,7 +18,7 @@ struct Relu2Mlp : FeedForward {
     if (host->take(ctx, M, inner, ctx->dtype, &act)) return 1;
     EngLinear up = {};
     up.out = act, up.a = x, up.w = up_w, up.gelu = 2;  // (activation code 2: the squared ReLU)
-    if (host->linear(ctx, &up, &ctx->pending)) return 1;
+    if (host->linear(ctx, &up, nullptr)) return 1;  // (nothing of this product may stay pending)
     EngLinear down = {};
     down.out = y, down.a.m = act, down.w = down_w, down.accumulate = overwrite ? 0 : 1;
     return host->linear(ctx, &down, &ctx->pending);

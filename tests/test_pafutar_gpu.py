@@ -143,15 +143,16 @@ def test_rmsnorm_kernel(width):
         assert (out.double().cpu() - want).abs().max() <= tol * want.abs().max()
 
 
+@pytest.mark.parametrize("W", [72, 70, 1280])  # (70: no multiple of four, the kernels for any width)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_token_shift_and_the_sum_that_is_normed(dtype):
+def test_token_shift_and_the_sum_that_is_normed(dtype, W):
     """Two requests' rows side by side: the shift reads the row before (the state for a portion's
     first row), the fused sum-and-norm keeps each request's last old row in the state."""
     import ctypes
 
     L = _ctypes_lib("post_norm_block")
     P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
-    W, g = 72, torch.Generator().manual_seed(1)
+    g = torch.Generator().manual_seed(1)
     h = torch.randn(7, W, generator=g).cuda()
     mu, s, gamma = (torch.rand(W, generator=g).cuda() for _ in range(3))
     state = torch.randn(4, W, generator=g).cuda()
@@ -166,10 +167,19 @@ def test_token_shift_and_the_sum_that_is_normed(dtype):
     y = torch.randn(7, W, generator=g).cuda()
     copy_ = torch.empty(7, W, dtype=dtype, device="cuda")
     h2 = h.clone()
-    assert L.residual_rmsnorm(P(h2), W, P(y), W, ctypes.c_float(1.5), P(s), P(gamma), ctypes.c_float(1e-4), P(state),
+    assert L.residual_rmsnorm(P(h2), W, P(y), W, None, 0, ctypes.c_float(1.5), P(s), P(gamma), ctypes.c_float(1e-4), P(state),
                               ctypes.c_size_t(W), P(slot_ids), P(token_req), P(copy_), code, 7, W, _stream()) == 0
     want = plain.rms_norm(1.5 * hc + s.double().cpu() * y.double().cpu(), gamma.double().cpu(), 1e-4)
     assert (h2.double().cpu() - want).abs().max() <= 2e-6
+    # the sublayer's output still in parts (a product that split its inner size), with and without rows beside them
+    parts = torch.randn(5, 7, W, generator=g).cuda()
+    for rows in (y, None):
+        h3 = h.clone()
+        assert L.residual_rmsnorm(P(h3), W, P(rows), W, P(parts), 5, ctypes.c_float(1.5), P(s), P(gamma), ctypes.c_float(1e-4),
+                                  None, ctypes.c_size_t(0), None, None, None, 0, 7, W, _stream()) == 0
+        total = parts.double().cpu().sum(0) + (y.double().cpu() if rows is not None else 0)
+        want3 = plain.rms_norm(1.5 * hc + s.double().cpu() * total, gamma.double().cpu(), 1e-4)
+        assert (h3.double().cpu() - want3).abs().max() <= 4e-6
     assert (copy_.double().cpu() - want).abs().max() <= (2e-6 if code == 0 else 2e-2)
     assert torch.equal(state[2], h[2]) and torch.equal(state[0], h[6])  # the old rows, not the normed ones
     assert torch.equal(state[1].cpu(), sc[1].float()) and torch.equal(state[3].cpu(), sc[3].float())
