@@ -8,7 +8,8 @@
 //
 // Everything here is computed in 32-bit on the 32-bit stream.  Kernels:
 //  * token_shift: the mixer's input in the compute dtype (without mu: a plain conversion).
-//  * residual_rmsnorm: h <- N(alpha h + s * y) in place, a wave a row; on the way it can keep
+//  * residual_rmsnorm: h <- N(alpha h + s * y) in place (y as rows, or as the parts of a product
+//    that split its inner size, or both); on the way it can keep
 //    the old rows that end a request's portion in the state tensor (the shift of the next step
 //    reads them) and leave a copy of the new rows in the compute dtype for the product that
 //    reads them next.

@@ -2,29 +2,53 @@
 //   y = x / sqrt(mean(x^2) + eps) * gamma          (eps inside the root; gamma may be absent)
 // The mean of squares, the root and the scale are computed in 32-bit; the output is float or
 // bfloat16.  With `rows` given, output row r is made from input row rows[r] (the rows whose
-// logits are wanted).  A wave a row, the row read twice (the second time from the caches).
+// logits are wanted).  A block a row with the row in registers; a wave a row for odd widths.
 //
 // Also the native part that stands for such a norm in a model (engine_parts.h).
 #include "common.h"
 #include "engine_parts.h"
 
-template <typename T, int VEC>
+// A block a row, the row in registers (NV float4 a thread, width <= 1024 NV): one trip to memory.
+template <typename T, int NV>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ x, int ldx,
                                                       const int* __restrict__ rows, const float* __restrict__ gamma,
-                                                      float eps, int n_rows, int width) {
+                                                      float eps, int width) {
+  __shared__ float red[32];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * ldx;
+  float4 v[NV], g[NV];
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = min((tid + 256 * i) * 4, width - 4);
+    v[i] = *(const float4*)(xr + k);
+    g[i] = gamma ? *(const float4*)(gamma + k) : make_float4(1.f, 1.f, 1.f, 1.f);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    if ((tid + 256 * i) * 4 < width) q += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+  const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)width + eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    if (k >= width) continue;
+    T* o = out + (size_t)r * width + k;
+    o[0] = from_f32<T>(v[i].x * rstd * g[i].x), o[1] = from_f32<T>(v[i].y * rstd * g[i].y);
+    o[2] = from_f32<T>(v[i].z * rstd * g[i].z), o[3] = from_f32<T>(v[i].w * rstd * g[i].w);
+  }
+}
+
+// Any width and alignment: a wave a row, a column a lane at a time, the row read twice.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_any_kernel(T* __restrict__ out, const float* __restrict__ x, int ldx,
+                                                          const int* __restrict__ rows, const float* __restrict__ gamma,
+                                                          float eps, int n_rows, int width) {
   const int lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;  // whole waves leave; no barrier follows
   const float* xr = x + (size_t)(rows ? rows[r] : r) * ldx;
   float q = 0.f;
-  if (VEC == 4) {
-    for (int k = lane * 4; k < width; k += 256) {
-      const float4 v = *(const float4*)(xr + k);
-      q += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
-    }
-  } else {
-    for (int k = lane; k < width; k += 64) q += xr[k] * xr[k];
-  }
+  for (int k = lane; k < width; k += 64) q += xr[k] * xr[k];
   const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
   T* o = out + (size_t)r * width;
   for (int k = lane; k < width; k += 64) o[k] = from_f32<T>(xr[k] * rstd * (gamma ? gamma[k] : 1.f));
@@ -38,18 +62,31 @@ extern "C" int rmsnorm(void* out, const float* x, int ldx, const int* rows, cons
   if (width <= 0 || ldx < width) FAIL("rmsnorm: width %d, row stride %d", width, ldx);
   if (!out || !x) FAIL("rmsnorm: null pointer");
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("rmsnorm: unknown dtype code %d", out_dtype);
-  const bool vec = width % 4 == 0 && ldx % 4 == 0 && !((uintptr_t)x & 15);
-  dim3 grid((n_rows + 3) / 4), block(256);
-  if (out_dtype == DT_F32) {
-    if (vec)
-      hipLaunchKernelGGL((rmsnorm_kernel<float, 4>), grid, block, 0, stream, (float*)out, x, ldx, rows, gamma, eps, n_rows, width);
+  const int nv4 = (width / 4 + 255) / 256;
+  const int nv = nv4 <= 1 ? 1 : nv4 <= 2 ? 2 : nv4 <= 4 ? 4 : nv4 <= 8 ? 8 : 0;
+  const bool vec = nv > 0 && width % 4 == 0 && ldx % 4 == 0 && !(((uintptr_t)x | (uintptr_t)gamma) & 15);
+  if (vec) {
+#define LAUNCH(T, NV) \
+  hipLaunchKernelGGL((rmsnorm_kernel<T, NV>), dim3(n_rows), dim3(256), 0, stream, (T*)out, x, ldx, rows, gamma, eps, width)
+#define BY_VECTORS(T)            \
+  do {                           \
+    if (nv == 1) LAUNCH(T, 1);   \
+    else if (nv == 2) LAUNCH(T, 2); \
+    else if (nv == 4) LAUNCH(T, 4); \
+    else LAUNCH(T, 8);           \
+  } while (0)
+    if (out_dtype == DT_F32)
+      BY_VECTORS(float);
     else
-      hipLaunchKernelGGL((rmsnorm_kernel<float, 1>), grid, block, 0, stream, (float*)out, x, ldx, rows, gamma, eps, n_rows, width);
+      BY_VECTORS(bf16);
+#undef BY_VECTORS
+#undef LAUNCH
   } else {
-    if (vec)
-      hipLaunchKernelGGL((rmsnorm_kernel<bf16, 4>), grid, block, 0, stream, (bf16*)out, x, ldx, rows, gamma, eps, n_rows, width);
+    dim3 grid((n_rows + 3) / 4), block(256);
+    if (out_dtype == DT_F32)
+      hipLaunchKernelGGL(rmsnorm_any_kernel<float>, grid, block, 0, stream, (float*)out, x, ldx, rows, gamma, eps, n_rows, width);
     else
-      hipLaunchKernelGGL((rmsnorm_kernel<bf16, 1>), grid, block, 0, stream, (bf16*)out, x, ldx, rows, gamma, eps, n_rows, width);
+      hipLaunchKernelGGL(rmsnorm_any_kernel<bf16>, grid, block, 0, stream, (bf16*)out, x, ldx, rows, gamma, eps, n_rows, width);
   }
   CHECK_LAUNCH("rmsnorm");
   return 0;

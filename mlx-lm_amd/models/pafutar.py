@@ -60,13 +60,22 @@ class ModelArgs(BaseModelArgs):
             m = entry["mixer"]
             if m.get("vdim", m["dim"]) != m["dim"]:
                 raise ValueError(f"layer {i}: the values are the keys, so vdim {m['vdim']} must equal dim {m['dim']}")
-            j = entry.get("weights_of")
-            if j is not None:
-                if not (isinstance(j, int) and 0 <= j < len(self.layers)) or "weights_of" in self.layers[j]:
-                    raise ValueError(f"layer {i}: weights_of {j!r} must name a layer that has weights of its own")
+            if entry.get("weights_of") is not None:
+                j = self.weights_layer(i)
                 other = self.layers[j]
                 if any(entry.get(k) != other.get(k) for k in ("type", "mixer", "mlp")):
                     raise ValueError(f"layer {i} runs with layer {j}'s weights but is described differently")
+
+    def weights_layer(self, i):
+        """The layer whose tensors layer ``i`` runs with: itself, or where its ``weights_of`` leads."""
+        seen = set()
+        while self.layers[i].get("weights_of") is not None:
+            j = self.layers[i]["weights_of"]
+            if not (isinstance(j, int) and 0 <= j < len(self.layers)) or i in seen:
+                raise ValueError(f"layer {i}: weights_of {j!r} must lead to a layer that has weights of its own")
+            seen.add(i)
+            i = j
+        return i
 
     @property
     def eps(self):
@@ -96,7 +105,7 @@ class Model:
         def norm(name):
             return PartSpec("rmsnorm", {"width": D, "eps": eps, "weight_name": name})
 
-        own = [i for i, e in enumerate(args.layers) if "weights_of" not in e]  # the layers with tensors
+        own = [i for i, e in enumerate(args.layers) if e.get("weights_of") is None]  # the layers with tensors
         index = {i: n for n, i in enumerate(own)}
         layers = []
         for i in own:
@@ -119,7 +128,7 @@ class Model:
         # every entry of the config is a run, with a cache and a shift state of its own; a run with
         # ``weights_of`` is a second run of that layer
         n = len(args.layers)
-        schedule = [RunEntry(layer=index[e.get("weights_of", i)], cache=i, state=n + i) for i, e in enumerate(args.layers)]
+        schedule = [RunEntry(layer=index[args.weights_layer(i)], cache=i, state=n + i) for i in range(n)]
         return ModelPlan(
             width=D, vocab_size=args.vocab, max_positions=args.max_positions,
             embedding=PartSpec("token", {"vocab_size": args.vocab, "width": D, "weight_name": "embed",
@@ -149,7 +158,7 @@ class Model:
 
         t = {"embed": normal((args.vocab, D), 0.02), "pos": normal((args.max_positions, D), 0.02 * args.embedding_scale)}
         for i, entry in enumerate(args.layers):
-            if "weights_of" in entry:
+            if entry.get("weights_of") is not None:
                 continue
             p, m = f"l{i}.", entry["mixer"]
             qw, kw = m["heads"] * m["dim"], m.get("kv_heads", m["heads"]) * m["dim"]

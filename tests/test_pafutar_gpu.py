@@ -390,6 +390,22 @@ def test_greedy_generation_through_the_scheduler(models):
     assert [[int(t) for t in text.split()] for text in batch.texts] == want
 
 
+def test_command_line(models):
+    """``python -m mlx_lm_amd generate`` on a Pafutar folder: the tokens the plain side generates,
+    also with a small pool of pages that the windows free as they pass."""
+    folder, config, weights = models["A"]
+    prompt = [3, 1, 4, 1, 5, 9, 2, 6]
+    want = _greedy(weights, config, prompt, 40)
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    for extra in ([], ["--num-pages", "6", "--prefill-step-size", "3"]):
+        out = subprocess.run(
+            [sys.executable, "-m", "mlx_lm_amd", "generate", "--model", folder, "--prompt-ids", ",".join(map(str, prompt)),
+             "--max-tokens", "40", "--dtype", "float32", "--verbose", "F"] + extra,
+            capture_output=True, text=True, env=env, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        assert out.stdout.strip() == " ".join(map(str, want))
+
+
 def test_trace_replay_of_a_random_model(tmp_path, models):
     """The replay program on a configuration with seeded random weights: logits files per step."""
     _, config, _ = models["A"]
