@@ -95,7 +95,9 @@ def relu_squared_ff(x, w, prefix):
 def layer(x, w, config, index):
     """One layer run; returns the stream after it."""
     entry = config["layers"][index]
-    src = entry.get("weights_of", index)
+    src = index
+    while config["layers"][src].get("weights_of") is not None:  # (a run may name a run that names a layer)
+        src = config["layers"][src]["weights_of"]
     p = f"l{src}."
     eps, alpha = config["norm"]["eps"], config["postln_alpha"]
     if entry["type"] != "attention":
@@ -136,7 +138,7 @@ def random_weights(config, seed, sharp=1.0):
 
     t = {"embed": normal((V, D), 0.05), "pos": normal((config["max_positions"], D), 0.3)}
     for i, entry in enumerate(config["layers"]):
-        if "weights_of" in entry:
+        if entry.get("weights_of") is not None:
             continue
         p, m = f"l{i}.", entry["mixer"]
         qw, kw = m["heads"] * m["dim"], m["kv_heads"] * m["dim"]

@@ -56,7 +56,15 @@ CONFIGS = {
     "F": _config(128, 300, [_layer(_mixer(2, 1, 64, window=70, keep_first=9), 256), _layer(_mixer(2, 2, 128, window=50, keep_first=33), 128),
                             _layer(_mixer(4, 2, 32), 64)], max_positions=512, alpha=2.0, scale=11.0),
 }
-SEEDS = {"A": 3, "B": 4, "F": 5}
+# the corners: one head, a head size beyond what the row kernels take and the smallest one, a window
+# of one token, more kept tokens than the window is long, a window and kept tokens that no sequence
+# here outgrows, a width that is no multiple of 64, a layer that runs three times
+CONFIGS["X"] = _config(72, 97, [_layer(_mixer(1, 1, 160, window=1, keep_first=0), 24), _layer(_mixer(3, 1, 8, window=5, keep_first=40)),
+                                _layer(_mixer(1, 1, 160, window=1, keep_first=0), 24, weights_of=0),
+                                _layer(_mixer(2, 2, 40, window=250, keep_first=300), 80),
+                                _layer(_mixer(1, 1, 160, window=1, keep_first=0), 24, weights_of=2)],
+                       max_positions=320, alpha=0.7, scale=0.5, eps=1e-3)
+SEEDS = {"A": 3, "B": 4, "F": 5, "X": 6}
 
 
 def _folder(path, config, weights):
@@ -251,7 +259,7 @@ def test_the_plain_side_notices_a_window_a_kept_token_and_a_shift(models, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,n", [("A", 200), ("B", 150), ("F", 300)])
+@pytest.mark.parametrize("name,n", [("A", 200), ("B", 150), ("F", 300), ("X", 310)])
 def test_whole_decoded_and_portions(models, dtype, name, n):
     folder, config, weights = models[name]
     tokens = helpers.random_tokens(n, config["vocab"], seed=n)
@@ -313,7 +321,7 @@ def test_windows_give_pages_back_and_stale_pages_do_not_matter(models, page_size
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "F"])
+@pytest.mark.parametrize("name", ["A", "B", "F", "X"])
 def test_mixed_batches_equal_each_request_alone(models, dtype, name):
     """Up to four live requests of unequal lengths, portions beside single tokens, requests that
     sit a step out; slots and pages of finished requests are used again by later ones."""
