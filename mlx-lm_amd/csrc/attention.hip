@@ -109,6 +109,27 @@ __device__ __forceinline__ void stage_tile(float* dst, int dst_stride, const T* 
                                            const int* table, const AttnArgs& p, int kv_head, int kt,
                                            int lo, int hi, int tid, int n_threads) {
   constexpr int VN = Vec<T>::N;
+  if (p.head_dim % VN != 0) {
+    // a head of bfloat16 that is a multiple of 4 only: 8-byte pieces
+    const int chunks = p.head_dim / 4;
+    const int total = KT * chunks;
+    for (int c = tid; c < total; c += n_threads) {
+      const int key = c / chunks, part = c - key * chunks;
+      const int pos = kt + key;
+      float f[4] = {0.f, 0.f, 0.f, 0.f};
+      if (pos >= lo && pos < hi) {
+        const int page = table[pos / p.page_size];
+        const T* src = pages + (size_t)page * p.page_stride +
+                       ((size_t)kv_head * p.page_size + (pos % p.page_size)) * p.head_dim + part * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = to_f32(src[i]);
+      }
+      float* d = dst + key * dst_stride + part * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = f[i];
+    }
+    return;
+  }
   const int chunks = p.head_dim / VN;
   const int total = KT * chunks;
   for (int c = tid; c < total; c += n_threads) {
@@ -604,8 +625,8 @@ static int check_geometry(const char* who, int n_heads, int n_kv_heads, int head
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("%s: unknown dtype code %d", who, dtype);
   if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
     FAIL("%s: %d query heads cannot be grouped over %d key heads", who, n_heads, n_kv_heads);
-  if (head_dim < 8 || head_dim > 256 || head_dim % 8 != 0)
-    FAIL("%s: head_dim %d must be a multiple of 8 between 8 and 256", who, head_dim);
+  if (head_dim < 4 || head_dim > 256 || head_dim % 4 != 0)
+    FAIL("%s: head_dim %d must be a multiple of 4 between 4 and 256", who, head_dim);
   if (page_size <= 0) FAIL("%s: page_size %d must be positive", who, page_size);
   return 0;
 }

@@ -16,7 +16,7 @@ extern "C" {
 #endif
 
 #define ENG_MAX_ARRAYS 32  // named integer arrays (and scalars) that parts ask the packer for
-#define ENG_MAX_GROUPS 8   // cache groups (block tables) a step can carry
+#define ENG_MAX_GROUPS 16  // cache groups (block tables) a step can carry
 
 // A matrix with contiguous rows on the device.  dtype: 0 float32, 1 bfloat16, 2 int32.
 typedef struct {

@@ -18,7 +18,7 @@ import torch
 from . import build
 
 MAX_ARRAYS = 32
-MAX_GROUPS = 8
+MAX_GROUPS = 16
 
 DT = {torch.float32: 0, torch.bfloat16: 1, torch.int32: 2}
 TORCH_DT = {0: torch.float32, 1: torch.bfloat16, 2: torch.int32}

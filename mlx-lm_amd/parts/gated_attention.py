@@ -36,10 +36,10 @@ class GatedKeyAttention(Mixer):
         n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} query heads cannot be grouped over {n_kv_heads} key heads")
-        if head_dim % 8 or not (8 <= head_dim <= 256):
-            raise ValueError(f"head_dim {head_dim} must be a multiple of 8 between 8 and 256")
-        if width % 8:
-            raise ValueError(f"width {width} must be a multiple of 8")
+        if head_dim % 4 or not (4 <= head_dim <= 256):
+            raise ValueError(f"head_dim {head_dim} must be a multiple of 4 between 4 and 256")
+        if width % 8 or (n_heads * head_dim) % 8:
+            raise ValueError(f"width {width} and the heads' columns {n_heads * head_dim} must be multiples of 8")
         if window < 0 or keep_first < 0:
             raise ValueError(f"window {window} and keep_first {keep_first} must not be negative")
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim

@@ -575,12 +575,12 @@ def test_attn_refuses_bad_head_dim():
     k = _k()
     from mlx_lm_amd.ops.kernels import PagedKV
 
-    pool = torch.zeros(4, 2, 1, 16, 20, device=DEV)
+    pool = torch.zeros(4, 2, 1, 16, 18, device=DEV)
     kv = PagedKV(pool[:, 0], pool[:, 1])
-    q = torch.zeros(1, 20, device=DEV)
+    q = torch.zeros(1, 18, device=DEV)
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
     bt = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
-    with pytest.raises(RuntimeError, match="multiple of 8"):
+    with pytest.raises(RuntimeError, match="multiple of 4"):
         k.attn_row(q.clone(), q, kv, bt, z, z, z, 1, 1, 1.0)
 
 

@@ -56,15 +56,20 @@ CONFIGS = {
     "F": _config(128, 300, [_layer(_mixer(2, 1, 64, window=70, keep_first=9), 256), _layer(_mixer(2, 2, 128, window=50, keep_first=33), 128),
                             _layer(_mixer(4, 2, 32), 64)], max_positions=512, alpha=2.0, scale=11.0),
 }
-# the corners: one head, a head size beyond what the row kernels take and the smallest one, a window
+# the corners: one head, a head size beyond what the row kernels take, small ones (8; 20 and 12,
+# multiples of four only), a window
 # of one token, more kept tokens than the window is long, a window and kept tokens that no sequence
 # here outgrows, a width that is no multiple of 64, a layer that runs three times
 CONFIGS["X"] = _config(72, 97, [_layer(_mixer(1, 1, 160, window=1, keep_first=0), 24), _layer(_mixer(3, 1, 8, window=5, keep_first=40)),
                                 _layer(_mixer(1, 1, 160, window=1, keep_first=0), 24, weights_of=0),
                                 _layer(_mixer(2, 2, 40, window=250, keep_first=300), 80),
+                                _layer(_mixer(2, 1, 20, window=30, keep_first=4), 16), _layer(_mixer(2, 2, 12)),
                                 _layer(_mixer(1, 1, 160, window=1, keep_first=0), 24, weights_of=2)],
                        max_positions=320, alpha=0.7, scale=0.5, eps=1e-3)
 SEEDS = {"A": 3, "B": 4, "F": 5, "X": 6}
+# how peaked the attention is: with seven layers as peaked as the others', bfloat16 rounding alone
+# moves a logit of X by 6 % now and then (any six of its layers: 2 to 3 %)
+SHARP = {"A": 4.0, "B": 4.0, "F": 4.0, "X": 1.5}
 
 
 def _folder(path, config, weights):
@@ -80,7 +85,7 @@ def _folder(path, config, weights):
 def models(tmp_path_factory):
     out = {}
     for name, config in CONFIGS.items():
-        weights = plain.random_weights(config, SEEDS[name], sharp=4.0)
+        weights = plain.random_weights(config, SEEDS[name], sharp=SHARP[name])
         out[name] = (_folder(str(tmp_path_factory.mktemp("paf" + name)), config, weights), config, weights)
     return out
 
