@@ -116,7 +116,10 @@ struct GatedKeyAttention : Mixer {
   fn_attn_decode_biased attn_decode = nullptr;
   fn_error attn_error = nullptr, prefill_error = nullptr, decode_error = nullptr;
 
-  GatedKeyAttention() { can_overwrite = true; }
+  typedef int (*fn_wants_packed)(const EngCtx*, const EngWeight*, int);
+  fn_wants_packed wants_packed = nullptr;
+
+  GatedKeyAttention() { can_overwrite = true, accepts_packed = true; }
 
   int kernels() {
     if (!attn_tile) {
@@ -183,8 +186,22 @@ struct GatedKeyAttention : Mixer {
       return host->fail("%s", g_err);
     host->launched(ctx);
 
+    const int n_tiles_ = (int)ctx->counts[array_base + ARR_TILES] / 2;
+    const int n_rows_ = (int)ctx->counts[array_base + ARR_ROWS];
+    const int key_bytes_ = head_dim * (ctx->dtype == DT_BF16 ? 2 : 4);
+    // Where every row goes to the kernel that streams keys through registers, that kernel writes
+    // the packed order (tiles of 16 rows x 64 columns) if the output product reads it faster so.
+    if (!wants_packed) wants_packed = (fn_wants_packed)host->kernel("engine", "eng_wants_packed_rows");
+    const bool pack = ctx->dtype == DT_BF16 && n_tiles_ == 0 && n_rows_ == T && head_dim <= ROW_KERNEL_MAX_HEAD_DIM &&
+                      (key_bytes_ == 64 || key_bytes_ == 128 || key_bytes_ == 256) && kv.page_size % (1024 / key_bytes_) == 0 &&
+                      wants_packed && wants_packed(ctx, &out_w, T);
     EngMat o;
-    if (host->take(ctx, T, q_width, ctx->dtype, &o)) return 1;
+    if (pack) {
+      if (host->take(ctx, (T + 15) / 16 * 16, (q_width + 63) / 64 * 64, DT_BF16, &o)) return 1;
+      o.rows = T, o.cols = q_width, o.ld = 0;
+    } else if (host->take(ctx, T, q_width, ctx->dtype, &o)) {
+      return 1;
+    }
     const char* gate = (const char*)qkg.p + (size_t)(q_width + kv_width) * (ctx->dtype == DT_BF16 ? 2 : 4);
     const int* tiles = ctx->arrays[array_base + ARR_TILES];
     const int* rows = ctx->arrays[array_base + ARR_ROWS];
@@ -258,7 +275,7 @@ struct GatedKeyAttention : Mixer {
       }
     }
     EngLinear out = {};
-    out.out = y, out.a.m = o, out.w = out_w, out.accumulate = overwrite ? 0 : 1;
+    out.out = y, out.a.m = o, out.a.packed = pack ? 1 : 0, out.w = out_w, out.accumulate = overwrite ? 0 : 1;
     return host->linear(ctx, &out, &ctx->pending);
   }
 };

@@ -25,7 +25,8 @@ __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out, c
                                                           const float* __restrict__ mu,
                                                           const float* __restrict__ state, size_t state_stride,
                                                           const int* __restrict__ slot_ids,
-                                                          const int* __restrict__ token_req, int width) {
+                                                          const int* __restrict__ token_req, int width,
+                                                          int packed_kblocks) {
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* xr = x + (size_t)r * ldx;
   const float* prev = xr;
@@ -50,7 +51,8 @@ __global__ __launch_bounds__(256) void token_shift_kernel(T* __restrict__ out, c
       o[0] += (pv[i].x - v[i].x) * m[i].x, o[1] += (pv[i].y - v[i].y) * m[i].y;
       o[2] += (pv[i].z - v[i].z) * m[i].z, o[3] += (pv[i].w - v[i].w) * m[i].w;
     }
-    T* at = out + (size_t)r * width + k;
+    // (packed_kblocks > 0: the order of packed_at, in which four columns from a multiple of four on stay together)
+    T* at = out + (packed_kblocks > 0 ? packed_at(r, k, packed_kblocks) : (size_t)r * width + k);
 #pragma unroll
     for (int c = 0; c < 4; ++c) at[c] = from_f32<T>(o[c]);
   }
@@ -67,7 +69,8 @@ __global__ __launch_bounds__(256) void residual_rmsnorm_kernel(float* __restrict
                                                                float* __restrict__ state, size_t state_stride,
                                                                const int* __restrict__ slot_ids,
                                                                const int* __restrict__ token_req,
-                                                               T* __restrict__ copy, int n_rows, int width) {
+                                                               T* __restrict__ copy, int n_rows, int width,
+                                                               int packed_kblocks) {
   __shared__ float red[32];
   const int r = blockIdx.x, tid = threadIdx.x;
   float* hr = h + (size_t)r * ldh;
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(256) void residual_rmsnorm_kernel(float* __restrict
                                  out[i].w * rstd * g[i].w);
     *(float4*)(hr + k) = n;
     if (copy) {
-      T* at = copy + (size_t)r * width + k;
+      T* at = copy + (packed_kblocks > 0 ? packed_at(r, k, packed_kblocks) : (size_t)r * width + k);
       at[0] = from_f32<T>(n.x), at[1] = from_f32<T>(n.y), at[2] = from_f32<T>(n.z), at[3] = from_f32<T>(n.w);
     }
   }
@@ -206,11 +209,16 @@ static inline int vectors_for(int width) {
     else LAUNCH(8);            \
   } while (0)
 
+// Whether the kernels that hold a row in registers take this width (they alone write the packed order).
+extern "C" int post_norm_rows_in_registers(int width) { return width % 4 == 0 && vectors_for(width) > 0; }
+
 // out [n_rows, width] (out_dtype) = shift(x); mu null: a conversion.  state [slots, state_stride] float32.
+// out_packed: a bfloat16 out in tiles of 16 rows x 64 columns, the order of packed_at (common.h).
 extern "C" int token_shift(void* out, const float* x, int ldx, const float* mu, const float* state,
                            size_t state_stride, const int* slot_ids, const int* token_req, int n_rows, int width,
-                           int out_dtype, hipStream_t stream) {
+                           int out_dtype, int out_packed, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  const int kblocks = out_packed ? (width + 63) / 64 : 0;
   if (width <= 0 || ldx < width) FAIL("token_shift: width %d, row stride %d", width, ldx);
   if (!out || !x) FAIL("token_shift: null pointer");
   if (mu && (!state || !slot_ids || !token_req || state_stride < (size_t)width))
@@ -219,14 +227,15 @@ extern "C" int token_shift(void* out, const float* x, int ldx, const float* mu, 
   const int nv = vectors_for(width);
   const bool vec = nv > 0 && width % 4 == 0 && ldx % 4 == 0 && state_stride % 4 == 0 && aligned16(x) && aligned16(mu) &&
                    aligned16(state);
+  if (out_packed && (!vec || out_dtype != DT_BF16)) FAIL("token_shift: the packed order is for bfloat16 rows that fit the registers");
   if (vec) {
 #define LAUNCH(NV)                                                                                                     \
   if (out_dtype == DT_F32)                                                                                             \
     hipLaunchKernelGGL((token_shift_kernel<float, NV>), dim3(n_rows), dim3(256), 0, stream, (float*)out, x, ldx, mu,  \
-                       state, state_stride, slot_ids, token_req, width);                                              \
+                       state, state_stride, slot_ids, token_req, width, 0);                                           \
   else                                                                                                                 \
     hipLaunchKernelGGL((token_shift_kernel<bf16, NV>), dim3(n_rows), dim3(256), 0, stream, (bf16*)out, x, ldx, mu,    \
-                       state, state_stride, slot_ids, token_req, width)
+                       state, state_stride, slot_ids, token_req, width, kblocks)
     BY_VECTORS(nv, LAUNCH);
 #undef LAUNCH
   } else {
@@ -250,8 +259,9 @@ extern "C" int token_shift(void* out, const float* x, int ldx, const float* mu, 
 extern "C" int residual_rmsnorm(float* h, int ldh, const float* y, int ldy, const float* parts, int n_parts,
                                 float alpha, const float* s, const float* gamma, float eps, float* state,
                                 size_t state_stride, const int* slot_ids, const int* token_req, void* copy,
-                                int copy_dtype, int n_rows, int width, hipStream_t stream) {
+                                int copy_dtype, int copy_packed, int n_rows, int width, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  const int kblocks = copy && copy_packed ? (width + 63) / 64 : 0;
   if (width <= 0 || ldh < width || (y && ldy < width)) FAIL("residual_rmsnorm: width %d, row strides %d and %d", width, ldh, ldy);
   if (!h || (!y && !parts)) FAIL("residual_rmsnorm: null pointer");
   if (!parts) n_parts = 0;
@@ -263,16 +273,17 @@ extern "C" int residual_rmsnorm(float* h, int ldh, const float* y, int ldy, cons
   const int nv = vectors_for(width);
   const bool vec = nv > 0 && width % 4 == 0 && ldh % 4 == 0 && ldy % 4 == 0 && state_stride % 4 == 0 && aligned16(h) &&
                    aligned16(y) && aligned16(parts) && aligned16(s) && aligned16(gamma) && aligned16(state);
+  if (kblocks && (!vec || !half)) FAIL("residual_rmsnorm: the packed order is for a bfloat16 copy of rows that fit the registers");
   if (vec) {
 #define LAUNCH(NV)                                                                                                       \
   if (half)                                                                                                              \
     hipLaunchKernelGGL((residual_rmsnorm_kernel<bf16, NV>), dim3(n_rows), dim3(256), 0, stream, h, ldh, y, ldy, parts,   \
                        n_parts, alpha, s, gamma, eps, state, state_stride, slot_ids, token_req, (bf16*)copy, n_rows,    \
-                       width);                                                                                          \
+                       width, kblocks);                                                                                 \
   else                                                                                                                   \
     hipLaunchKernelGGL((residual_rmsnorm_kernel<float, NV>), dim3(n_rows), dim3(256), 0, stream, h, ldh, y, ldy, parts,  \
                        n_parts, alpha, s, gamma, eps, state, state_stride, slot_ids, token_req, (float*)copy, n_rows,   \
-                       width)
+                       width, 0)
     BY_VECTORS(nv, LAUNCH);
 #undef LAUNCH
   } else {
@@ -322,6 +333,23 @@ struct PostNormBlock : Block {
     return 0;
   }
 
+  // Whether the product of n_rows rows with w reads its rows faster in the packed order (the
+  // host's answer), and the rows' own kernels here can write it.
+  typedef int (*fn_wants_packed)(const EngCtx*, const EngWeight*, int);
+  fn_wants_packed host_wants_packed = nullptr;
+  bool wants_packed(EngCtx* ctx, int n_rows, const EngWeight* w) {
+    if (!w || ctx->dtype != DT_BF16 || !post_norm_rows_in_registers(width)) return false;
+    if (!host_wants_packed) host_wants_packed = (fn_wants_packed)host->kernel("engine", "eng_wants_packed_rows");
+    return host_wants_packed && host_wants_packed(ctx, w, n_rows) != 0;
+  }
+  // Rows of the compute dtype for a product: row-major, or whole tiles of 16 rows x 64 columns.
+  int take_rows(EngCtx* ctx, int n_rows, bool packed, EngValue* out) {
+    if (!packed) return host->take(ctx, n_rows, width, ctx->dtype, &out->m);
+    if (host->take(ctx, (n_rows + 15) / 16 * 16, (width + 63) / 64 * 64, DT_BF16, &out->m)) return 1;
+    out->m.rows = n_rows, out->m.cols = width, out->m.ld = 0, out->packed = 1;
+    return 0;
+  }
+
   int zero(EngCtx* ctx, const EngMat& y) {
     const size_t n = (size_t)y.rows * y.ld;
     hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, (float*)y.p, n);
@@ -347,9 +375,11 @@ struct PostNormBlock : Block {
     // what the mixer reads
     EngValue u = {};
     if (mu || ctx->dtype != DT_F32 || h.ld != width) {
-      if (host->take(ctx, T, width, ctx->dtype, &u.m)) return 1;
+      // (in the packed order where the mixer's first product reads its rows faster so)
+      const bool pack = mixer->accepts_packed && wants_packed(ctx, T, mixer->first_weight);
+      if (take_rows(ctx, T, pack, &u)) return 1;
       if (token_shift(u.m.p, (const float*)h.p, h.ld, mu, state, state_stride, ctx->slot_ids, ctx->token_req, T, width,
-                      ctx->dtype, ctx->stream))
+                      ctx->dtype, pack ? 1 : 0, ctx->stream))
         return host->fail("%s", g_err);
       host->launched(ctx);
     } else {
@@ -373,11 +403,11 @@ struct PostNormBlock : Block {
     EngValue x = {};
     x.m = h;
     if (ffn && ctx->dtype != DT_F32) {
-      if (host->take(ctx, T, width, ctx->dtype, &x.m)) return 1;
+      if (take_rows(ctx, T, ffn->accepts_packed && wants_packed(ctx, T, ffn->first_weight), &x)) return 1;
     }
     if (residual_rmsnorm((float*)h.p, h.ld, parts.y, y.ld, parts.ws, parts.n, alpha, scale1, gamma1, eps, state,
-                         state_stride, ctx->slot_ids, ctx->token_req, x.m.p != h.p ? x.m.p : nullptr, ctx->dtype, T, width,
-                         ctx->stream))
+                         state_stride, ctx->slot_ids, ctx->token_req, x.m.p != h.p ? x.m.p : nullptr, ctx->dtype, x.packed, T,
+                         width, ctx->stream))
       return host->fail("%s", g_err);
     host->launched(ctx);
     if (ffn) {
@@ -388,7 +418,7 @@ struct PostNormBlock : Block {
       if (rc) return rc;
       if (take_parts(ctx, y, !ffn->overwrite, &parts)) return 1;
       if (residual_rmsnorm((float*)h.p, h.ld, parts.y, y.ld, parts.ws, parts.n, alpha, scale2, gamma2, eps, nullptr, 0,
-                           nullptr, nullptr, nullptr, 0, T, width, ctx->stream))
+                           nullptr, nullptr, nullptr, 0, 0, T, width, ctx->stream))
         return host->fail("%s", g_err);
       host->launched(ctx);
     }
