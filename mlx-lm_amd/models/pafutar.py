@@ -117,7 +117,7 @@ class Model:
             parts = dict(
                 mixer=PartSpec("gated_key_attention", {
                     "width": D, "n_heads": m["heads"], "n_kv_heads": m.get("kv_heads", m["heads"]),
-                    "head_dim": m["dim"], "scale": m["scale"], "window": window,
+                    "head_dim": m["dim"], "scale": m.get("scale", m["dim"] ** -0.5), "window": window,
                     "keep_first": int(mask.get("keep_first", 0)), "eps": eps}, p + "mix."),
                 mixer_norm=norm(p + "norm1"))
             if entry.get("mlp") is not None:

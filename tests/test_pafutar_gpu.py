@@ -393,6 +393,65 @@ def test_twenty_requests_decode_together(models, dtype, name):
         _close(torch.stack(got[i]), _plain(weights, config, tokens[i], dtype)[n:], dtype, f"request {i} among twenty")
 
 
+def _drawn_config(seed):
+    """A configuration drawn from the seed: every size, the layers' order, windows and constants."""
+    g = torch.Generator().manual_seed(seed)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (), generator=g))]
+
+    own = []
+    for _ in range(pick([1, 2, 3])):
+        kv_heads = pick([1, 2, 3])
+        heads = kv_heads * pick([1, 2, 4])
+        dim = pick([4, 8, 12, 16, 24, 32, 40, 64, 72, 128, 160])
+        if (heads * dim) % 8:
+            dim *= 2
+        window = pick([None, 1, 7, 16, 33, 64, 100, 1000])
+        keep = pick([0, 0, 1, 5, 16, 17, 50]) if window else 0
+        own.append(_layer(_mixer(heads, kv_heads, dim, window, keep, scale=pick([None, 0.05, 0.4])), pick([None, 8, 44, 96, 200])))
+    layers = list(own)
+    for _ in range(pick([0, 1, 3])):
+        j = pick(list(range(len(own))))
+        layers.insert(pick(list(range(len(own), len(layers) + 1))), dict(copy.deepcopy(own[j]), weights_of=j))
+    return _config(pick([16, 40, 64, 104, 256]), pick([17, 100, 257, 1000]), layers, max_positions=pick([160, 200, 512]),
+                   alpha=pick([0.5, 1.0, 2.5, 4.0]), scale=pick([1.0, 8.0, 0.3]), eps=pick([1e-6, 1e-5, 1e-2]))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_configurations(tmp_path, seed):
+    """Ten drawn configurations (layers of several shapes in one model, so several cache groups;
+    layers run again with a cache of their own) in mixed batches with few pages, against each
+    request alone on the plain side: float32 all, bfloat16 every other one."""
+    from mlx_lm_amd.engine import StepEntry
+
+    config = _drawn_config(seed)
+    weights = plain.random_weights(config, 50 + seed, sharp=2.0)
+    folder = _folder(str(tmp_path / "m"), config, weights)
+    lengths = [n for n in [70, 9, 131, 40, 3, 97] if n <= config["max_positions"]]
+    tokens, steps = helpers.mixed_trace({"vocab_size": config["vocab"]}, seed, lengths, n_live=3)
+    for dtype in ["float32"] + (["bfloat16"] if seed % 2 == 0 else []):
+        eng = _engine(folder, dtype, n_pages=helpers.held(lengths, 3) // 16, max_requests=3)
+        got = {rid: [] for rid in tokens}
+        for s in steps:
+            entries = []
+            for e in s["entries"]:
+                if not eng.has_request(e["id"]):
+                    eng.add_request(e["id"])
+                entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+            logits = eng.step(entries).clone()
+            at = 0
+            for e in entries:
+                got[e.request_id].append(logits[at : at + len(e.want)])
+                at += len(e.want)
+            for rid in s["end"]:
+                eng.end_request(rid)
+            eng.cache.poison_free_pages()
+        for rid, toks in tokens.items():
+            _close(torch.cat(got[rid]), _plain(weights, config, toks, dtype), dtype, f"seed {seed}: request {rid} ({config['layers']})")
+        eng.cache.check()
+
+
 def test_recorded_steps_equal_eager_steps(models):
     """Decode steps replayed from recorded graphs against the same steps run eagerly, bit for bit
     (the shift's state is read and written once a step either way)."""
