@@ -452,6 +452,39 @@ def test_drawn_configurations(tmp_path, seed):
         eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_thousands_of_keys(tmp_path, dtype):
+    """A prompt of 3,300 tokens in two portions, then 40 decoded tokens beside a short request:
+    layers without a window (a decoded row's keys are split over blocks, in the kernel that
+    streams keys through registers and in the general one), a window of 1,500 that keeps 40, and
+    a short window far from the start.  (That a single far key counts is the kernels' own test.)"""
+    from mlx_lm_amd.engine import StepEntry
+
+    config = _config(64, 120, [_layer(_mixer(2, 1, 64), 48), _layer(_mixer(4, 2, 24, window=1500, keep_first=40)),
+                               _layer(_mixer(2, 2, 48)), _layer(_mixer(2, 1, 64, window=70, keep_first=130), 48)],
+                     max_positions=3400, alpha=1.3, scale=4.0)
+    weights = plain.random_weights(config, 31, sharp=3.0)
+    folder = _folder(str(tmp_path / "long"), config, weights)
+    n, n_prompt = 3340, 3300
+    tokens = helpers.random_tokens(n, config["vocab"], seed=31)
+    short = helpers.random_tokens(60, config["vocab"], seed=32)
+    want = _plain(weights, config, tokens, dtype)
+    eng = _engine(folder, dtype, n_pages=(n + 15) // 16 + 6)
+    eng.add_request("long")
+    eng.add_request("short")
+    rows = [eng.step([StepEntry("long", tokens[:2000], [1999])]).clone(),
+            eng.step([StepEntry("long", tokens[2000:n_prompt], [n_prompt - 2001]), StepEntry("short", short[:20], [])])[:1].clone()]
+    _close(torch.cat(rows), want[[1999, n_prompt - 1]], dtype, "the prompt's portions")
+    got, got_short = [], []
+    for i in range(n - n_prompt):
+        logits = eng.step([StepEntry("long", [tokens[n_prompt + i]], [0]), StepEntry("short", [short[20 + i]], [0])]).clone()
+        got.append(logits[0])
+        got_short.append(logits[1])
+    _close(torch.stack(got), want[n_prompt:], dtype, "decoding at 3,300 keys")
+    _close(torch.stack(got_short), _plain(weights, config, short, dtype)[20:], dtype, "the short request beside it")
+    assert eng.stats.key_splits_most > 1  # a row's keys did go over several blocks
+
+
 def test_recorded_steps_equal_eager_steps(models):
     """Decode steps replayed from recorded graphs against the same steps run eagerly, bit for bit
     (the shift's state is read and written once a step either way)."""
@@ -585,6 +618,8 @@ def test_attention_kernels_with_score_terms(kernel, dtype, d, window, keep_first
         for j, factor in edges:
             if 0 <= j < n:
                 k[j, G - 1] = (q[0, H - 1].float() * factor).to(dtype)
+    else:
+        k[2, G - 1] = (q[0, H - 1].float() * 1.8).to(dtype)  # one key far back, among hundreds
     slopes = plain.head_slopes(H).float()
     # the plain side: scores with scale 1 and the heads' temperatures, the mask, the gate
     s = plain.attention_scores(q.double(), k.double(), 1.0, temp.double(), offset)
@@ -594,6 +629,8 @@ def test_attention_kernels_with_score_terms(kernel, dtype, d, window, keep_first
     want = want * torch.sigmoid(gate.double())
     if window and keep_first:
         assert p[H - 1, 0, keep_first - 1] > 0.1  # the first query leans on the last kept key
+    if not window:
+        assert p[H - 1, 0, 2] > 0.1  # and on the far key
 
     kv, table = _paged(k, v, 16, dtype, seed=d)
     qd = q.reshape(n_q, H * d).cuda()
