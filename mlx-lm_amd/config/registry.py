@@ -6,7 +6,8 @@ import importlib
 MODEL_REMAPPING = {}
 
 _REGISTRY = {}
-_BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2", "pafutar": "mlx_lm_amd.models.pafutar"}
+_BUILTIN = {"gpt2": "mlx_lm_amd.models.gpt2", "pafutar": "mlx_lm_amd.models.pafutar",
+            "ruzolorn": "mlx_lm_amd.models.ruzolorn"}
 
 
 def register_model(model_type, model_cls, args_cls):

@@ -117,6 +117,7 @@ typedef struct {
   EngMat x, residual, out, q, k;
   const int* rows;
   int n_rows, cache_slot, writes_cache, lazy;
+  int state_slot, pad_;  // a block's second slot (per-request state of this run), or -1
   // results: a norm's output; an embedding term's table and index
   EngMat result;
   const int* index;

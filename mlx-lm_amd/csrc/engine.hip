@@ -600,9 +600,9 @@ struct PyFeedForward : FeedForward {
 struct PyBlock : Block {
   int id;
   PyBlock(int i, int flags) : id(i) { handles_pending = false, (void)flags; }
-  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int) override {
+  int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes, int state_slot) override {
     EngCall c = {};
-    c.residual = h, c.cache_slot = slot, c.writes_cache = writes;
+    c.residual = h, c.cache_slot = slot, c.writes_cache = writes, c.state_slot = state_slot;
     return call_python(id, ENG_CB_BLOCK, ctx, &c);
   }
 };

@@ -1,0 +1,272 @@
+// Mixers whose memory of a sequence is a matrix per head that decays and takes an outer product
+// at every token (linear attention with a decay, the selective state space with a scalar decay a
+// head), and the kernels around them:
+//
+//   state_scan      S_t = a_t S_(t-1) + k_t v_t^T,  o_t = S_t^T q_t  (+ skip_h v_t)
+//                   S is N x P (key size x value size), 32-bit, kept per request and head between
+//                   steps.  a_t = exp(log_a[t, h]) or the constant decay[h]; k_t is multiplied by
+//                   k_mult and by k_scale[t, h] where given; q and k may turn with the position
+//                   (the first rot_dims columns of a head, column i with column i + rot_dims / 2,
+//                   by position * inv_freq[i]); the key heads may be fewer than the value heads
+//                   (head h reads key head h / (H / Hk)).  The output may be divided by its root
+//                   mean square over the head and multiplied by silu(gate) on the way out.
+//   ssm_prepare     causal convolution per channel over a request's tokens with the last
+//                   taps - 1 inputs of earlier steps from the state, bias, silu; and the step
+//                   sizes: dt = softplus(raw + dt_bias), log_a = -exp(A_log) dt.
+//   conv_state_update  the last taps - 1 inputs of each request, for the next step.
+//   gated_group_rmsnorm  out = RMSnorm_in_groups(y * silu(z)) * w.
+//
+// Everything here is 32-bit: the operands arrive as float rows (the projections write float),
+// the state is float, angles, decays, exponentials and norms are float; only `out` of the scan
+// and of the gated norm may be bfloat16.  Sums run in a fixed order.
+#include "common.h"
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+struct ScanArgs {
+  const float* q;
+  const float* k;
+  const float* v;
+  int ldq, ldk, ldv;
+  const float* log_a;    // [tokens, H] or null
+  const float* decay;    // [H], where log_a is null
+  const float* k_scale;  // [tokens, H] or null
+  float k_mult;
+  const float* skip;  // [H] or null
+  int rot_dims;
+  const float* inv_freq;  // [rot_dims / 2]
+  const int* positions;   // [tokens]
+  int unit_rms;
+  float eps;
+  const float* gate;  // [tokens, ldg] or null, head h at column h * P
+  int ldg;
+  void* out;  // [tokens, ldo], head h at column h * P
+  int ldo, out_dtype;
+  float* state;  // request r, head h: state + slot_ids[r] * state_stride + state_offset + h * N * P
+  size_t state_stride, state_offset;
+  const int* seq_start;
+  const int* seq_len;
+  const int* slot_ids;
+  int n_requests, H, Hk, N, P;
+};
+
+// One block a (head, request); the state in LDS as S[i * P + p], thread (part, p) walks its share
+// of the keys i for value column p.  Tokens in turn: the recurrence as written.
+template <typename T>
+__global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
+  extern __shared__ float lds[];
+  __shared__ float red[32];
+  const int N = a.N, P = a.P, tid = threadIdx.x;
+  const int h = blockIdx.x, r = blockIdx.y, hk = h / (a.H / a.Hk);
+  const int parts = min(256 / P, N), chunk = (N + parts - 1) / parts;
+  float* S = lds;
+  float* qs = S + (size_t)N * P;
+  float* ks = qs + N;
+  float* vs = ks + N;
+  float* partial = vs + P;  // [parts, P]
+  const int start = a.seq_start[r], n = a.seq_len[r];
+  float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P;
+  for (int i = tid; i < N * P; i += 256) S[i] = Sg[i];
+  const int half = a.rot_dims / 2;
+  const int p = tid % P, part = tid / P;
+  const bool works = tid < parts * P;
+  const int i0 = part * chunk, i1 = min(N, i0 + chunk);
+  for (int t = 0; t < n; ++t) {
+    const size_t row = (size_t)(start + t);
+    __syncthreads();  // the token before is done with qs, ks, vs, partial (and S is loaded)
+    const float ksc = a.k_mult * (a.k_scale ? a.k_scale[row * a.H + h] : 1.0f);
+    for (int i = tid; i < N; i += 256) {
+      const float* qr = a.q + row * a.ldq + (size_t)hk * N;
+      const float* kr = a.k + row * a.ldk + (size_t)hk * N;
+      float qv = qr[i], kv = kr[i];
+      if (i < a.rot_dims) {
+        const int j = i < half ? i : i - half;
+        float sn, cs;
+        sincosf((float)a.positions[row] * a.inv_freq[j], &sn, &cs);
+        if (i < half)
+          qv = qr[j] * cs - qr[j + half] * sn, kv = kr[j] * cs - kr[j + half] * sn;
+        else
+          qv = qr[j + half] * cs + qr[j] * sn, kv = kr[j + half] * cs + kr[j] * sn;
+      }
+      qs[i] = qv, ks[i] = kv * ksc;
+    }
+    for (int c = tid; c < P; c += 256) vs[c] = a.v[row * a.ldv + (size_t)h * P + c];
+    const float at = a.log_a ? expf(a.log_a[row * a.H + h]) : a.decay[h];
+    __syncthreads();
+    if (works) {
+      const float vp = vs[p];
+      float acc = 0.f;
+      for (int i = i0; i < i1; ++i) {
+        const float s = at * S[(size_t)i * P + p] + ks[i] * vp;
+        S[(size_t)i * P + p] = s;
+        acc += s * qs[i];
+      }
+      partial[part * P + p] = acc;
+    }
+    __syncthreads();
+    float o = 0.f;
+    if (tid < P) {
+      for (int j = 0; j < parts; ++j) o += partial[j * P + tid];
+      if (a.skip) o += a.skip[h] * vs[tid];
+    }
+    if (a.unit_rms) {
+      const float ss = block_sum(tid < P ? o * o : 0.f, red);
+      o *= 1.0f / sqrtf(ss / (float)P + a.eps);
+    }
+    if (tid < P) {
+      if (a.gate) o *= silu_f(a.gate[row * a.ldg + (size_t)h * P + tid]);
+      ((T*)a.out)[row * a.ldo + (size_t)h * P + tid] = from_f32<T>(o);
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < N * P; i += 256) Sg[i] = S[i];
+}
+
+// ---------------------------------------------------------------------------
+
+// Thread (token row, channel c): c < C is a convolution channel, C <= c < C + H a head's step size.
+__global__ __launch_bounds__(256) void ssm_prepare_kernel(
+    const float* __restrict__ u, int ldu, int conv_col, int dt_col, const float* __restrict__ w,
+    const float* __restrict__ b, int taps, int C, int H, const float* __restrict__ dt_bias,
+    const float* __restrict__ A_log, const float* __restrict__ state, size_t state_stride, size_t conv_offset,
+    const int* __restrict__ token_req, const int* __restrict__ seq_start, const int* __restrict__ slot_ids,
+    float* __restrict__ xbc, float* __restrict__ dt, float* __restrict__ log_a, int n_tokens) {
+  const int c = blockIdx.y * 256 + threadIdx.x, row = blockIdx.x;
+  if (c >= C + H) return;
+  if (c >= C) {
+    const int hd = c - C;
+    const float d = softplus_f(u[(size_t)row * ldu + dt_col + hd] + dt_bias[hd]);
+    dt[(size_t)row * H + hd] = d;
+    log_a[(size_t)row * H + hd] = -expf(A_log[hd]) * d;
+    return;
+  }
+  const int req = token_req[row], local = row - seq_start[req];
+  const float* old = state + (size_t)slot_ids[req] * state_stride + conv_offset;  // [taps - 1, C], the latest last
+  float acc = b ? b[c] : 0.f;
+  for (int j = taps - 1; j >= 0; --j) {  // the oldest input first
+    const int at = local - j;
+    const float in = at >= 0 ? u[(size_t)(row - j) * ldu + conv_col + c] : old[(size_t)(taps - 1 + at) * C + c];
+    acc += w[(size_t)c * taps + (taps - 1 - j)] * in;
+  }
+  xbc[(size_t)row * C + c] = silu_f(acc);
+}
+
+// Thread (request, channel): the new last taps - 1 inputs, ascending, so that what is still to be
+// read of the old ones lies ahead of what is written.
+__global__ __launch_bounds__(256) void conv_state_update_kernel(const float* __restrict__ u, int ldu, int conv_col,
+                                                                int taps, int C, float* __restrict__ state,
+                                                                size_t state_stride, size_t conv_offset,
+                                                                const int* __restrict__ seq_start,
+                                                                const int* __restrict__ seq_len,
+                                                                const int* __restrict__ slot_ids) {
+  const int c = blockIdx.x * 256 + threadIdx.x, req = blockIdx.y;
+  if (c >= C) return;
+  const int start = seq_start[req], n = seq_len[req];
+  float* st = state + (size_t)slot_ids[req] * state_stride + conv_offset;
+  for (int j = 0; j < taps - 1; ++j) {
+    const int at = n - (taps - 1) + j;
+    st[(size_t)j * C + c] = at >= 0 ? u[(size_t)(start + at) * ldu + conv_col + c] : st[(size_t)(j + n) * C + c];
+  }
+}
+
+// A block a (row, group).
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* __restrict__ y, int ldy,
+                                                                  const float* __restrict__ z, int ldz,
+                                                                  const float* __restrict__ w, float eps, int size,
+                                                                  T* __restrict__ out, int ldo) {
+  __shared__ float red[32];
+  const int row = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+  const float* yr = y + (size_t)row * ldy + (size_t)g * size;
+  const float* zr = z + (size_t)row * ldz + (size_t)g * size;
+  float q = 0.f;
+  for (int k = tid; k < size; k += 256) {
+    const float s = yr[k] * silu_f(zr[k]);
+    q += s * s;
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(q, red) / (float)size + eps);
+  for (int k = tid; k < size; k += 256)
+    out[(size_t)row * ldo + (size_t)g * size + k] = from_f32<T>(yr[k] * silu_f(zr[k]) * rstd * w[(size_t)g * size + k]);
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+#define SCAN_MAX_LDS (152 * 1024)
+
+extern "C" int state_scan(const ScanArgs* args, hipStream_t stream) {
+  const ScanArgs& a = *args;
+  if (a.n_requests <= 0 || a.H <= 0) return 0;
+  if (!a.q || !a.k || !a.v || !a.out || !a.state || !a.seq_start || !a.seq_len || !a.slot_ids)
+    FAIL("state_scan: null pointer");
+  if (a.N <= 0 || a.P <= 0 || a.P > 256) FAIL("state_scan: key size %d, value size %d (at most 256)", a.N, a.P);
+  if (a.Hk <= 0 || a.H % a.Hk) FAIL("state_scan: %d heads over %d key heads", a.H, a.Hk);
+  if (!a.log_a && !a.decay) FAIL("state_scan: a decay per token or per head is needed");
+  if (a.rot_dims && (a.rot_dims % 2 || a.rot_dims > a.N || !a.inv_freq || !a.positions))
+    FAIL("state_scan: %d turning columns of %d", a.rot_dims, a.N);
+  if (a.ldq < a.Hk * a.N || a.ldk < a.Hk * a.N || a.ldv < a.H * a.P || a.ldo < a.H * a.P || (a.gate && a.ldg < a.H * a.P))
+    FAIL("state_scan: a row is narrower than its heads");
+  if (a.out_dtype != DT_F32 && a.out_dtype != DT_BF16) FAIL("state_scan: unknown dtype code %d", a.out_dtype);
+  const int parts = a.N < 256 / a.P ? a.N : 256 / a.P;
+  const size_t lds = ((size_t)a.N * a.P + 2 * (size_t)a.N + a.P + (size_t)parts * a.P) * sizeof(float);
+  if (lds > SCAN_MAX_LDS) FAIL("state_scan: a state of %d x %d does not fit a block's LDS", a.N, a.P);
+  static bool raised = false;
+  if (!raised) {
+    (void)hipFuncSetAttribute((const void*)state_scan_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+    (void)hipFuncSetAttribute((const void*)state_scan_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+    raised = true;
+  }
+  dim3 grid(a.H, a.n_requests), block(256);
+  if (a.out_dtype == DT_F32)
+    hipLaunchKernelGGL(state_scan_kernel<float>, grid, block, lds, stream, a);
+  else
+    hipLaunchKernelGGL(state_scan_kernel<bf16>, grid, block, lds, stream, a);
+  CHECK_LAUNCH("state_scan");
+  return 0;
+}
+
+extern "C" int ssm_prepare(const float* u, int ldu, int conv_col, int dt_col, const float* w, const float* b, int taps,
+                           int C, int H, const float* dt_bias, const float* A_log, const float* state,
+                           size_t state_stride, size_t conv_offset, const int* token_req, const int* seq_start,
+                           const int* slot_ids, float* xbc, float* dt, float* log_a, int n_tokens, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (!u || !w || !dt_bias || !A_log || !state || !token_req || !seq_start || !slot_ids || !xbc || !dt || !log_a)
+    FAIL("ssm_prepare: null pointer");
+  if (taps < 1 || C <= 0 || H <= 0 || conv_col < 0 || dt_col < 0 || conv_col + C > ldu || dt_col + H > ldu)
+    FAIL("ssm_prepare: %d taps, %d channels from column %d, %d heads from column %d, rows of %d", taps, C, conv_col, H, dt_col, ldu);
+  dim3 grid(n_tokens, (C + H + 255) / 256), block(256);
+  hipLaunchKernelGGL(ssm_prepare_kernel, grid, block, 0, stream, u, ldu, conv_col, dt_col, w, b, taps, C, H, dt_bias,
+                     A_log, state, state_stride, conv_offset, token_req, seq_start, slot_ids, xbc, dt, log_a, n_tokens);
+  CHECK_LAUNCH("ssm_prepare");
+  return 0;
+}
+
+extern "C" int conv_state_update(const float* u, int ldu, int conv_col, int taps, int C, float* state,
+                                 size_t state_stride, size_t conv_offset, const int* seq_start, const int* seq_len,
+                                 const int* slot_ids, int n_requests, hipStream_t stream) {
+  if (n_requests <= 0 || taps <= 1) return 0;
+  if (!u || !state || !seq_start || !seq_len || !slot_ids) FAIL("conv_state_update: null pointer");
+  if (C <= 0 || conv_col < 0 || conv_col + C > ldu) FAIL("conv_state_update: %d channels from column %d in rows of %d", C, conv_col, ldu);
+  dim3 grid((C + 255) / 256, n_requests), block(256);
+  hipLaunchKernelGGL(conv_state_update_kernel, grid, block, 0, stream, u, ldu, conv_col, taps, C, state, state_stride,
+                     conv_offset, seq_start, seq_len, slot_ids);
+  CHECK_LAUNCH("conv_state_update");
+  return 0;
+}
+
+extern "C" int gated_group_rmsnorm(const float* y, int ldy, const float* z, int ldz, const float* w, float eps,
+                                   int n_rows, int width, int groups, void* out, int ldo, int out_dtype,
+                                   hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (!y || !z || !w || !out) FAIL("gated_group_rmsnorm: null pointer");
+  if (groups <= 0 || width <= 0 || width % groups || ldy < width || ldz < width || ldo < width)
+    FAIL("gated_group_rmsnorm: width %d in %d groups, row strides %d, %d, %d", width, groups, ldy, ldz, ldo);
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("gated_group_rmsnorm: unknown dtype code %d", out_dtype);
+  dim3 grid(n_rows, groups), block(256);
+  if (out_dtype == DT_F32)
+    hipLaunchKernelGGL(gated_group_rmsnorm_kernel<float>, grid, block, 0, stream, y, ldy, z, ldz, w, eps, width / groups, (float*)out, ldo);
+  else
+    hipLaunchKernelGGL(gated_group_rmsnorm_kernel<bf16>, grid, block, 0, stream, y, ldy, z, ldz, w, eps, width / groups, (bf16*)out, ldo);
+  CHECK_LAUNCH("gated_group_rmsnorm");
+  return 0;
+}

@@ -22,7 +22,8 @@ _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(_PKG, "csrc")
 
 SOURCES = ("embed", "norm", "rmsnorm", "gemm_f32", "gemm_bf16", "gemm_bf16_decode", "attention", "attention_decode",
-           "attention_prefill", "gated_key_attention", "relu2_mlp", "post_norm_block", "sampling", "engine")
+           "attention_prefill", "gated_key_attention", "relu2_mlp", "post_norm_block", "sandwich_block", "head_norm",
+           "linear_state", "experts", "sampling", "engine")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

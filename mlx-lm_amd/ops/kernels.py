@@ -807,3 +807,248 @@ def apply_penalties(logits, offsets, hist, rep, rep_ctx, pres, pres_ctx, freq, f
                              _ptr(rep), _ptr(rep_ctx), _ptr(pres), _ptr(pres_ctx), _ptr(freq),
                              _ptr(freq_ctx), _c_int(logits.shape[1]), _stream())
     build.check(lib, rc, "apply_penalties")
+
+
+# ---------------------------------------------------------------------------
+# layers normed on both sides of their sublayers; heads normed one by one
+
+
+def add_normed(h, y, w_post, mult, eps, w_next=None, out=None):
+    """``h += mult * LN(y; w_post)`` on float32 rows, and ``out = LN(h; w_next)`` of the new rows
+    where ``w_next`` is given (csrc/sandwich_block.hip)."""
+    lib = build.load("sandwich_block")
+    ldh, ldy = _rows2d(h, "h"), _rows2d(y, "y")
+    _need(h.dtype == torch.float32 and y.dtype == torch.float32 and h.shape == y.shape, "add_normed: float32 rows of one shape")
+    n, width = h.shape
+    _dev(w_post, "w_post", torch.float32)
+    _need(w_post.numel() == width, "add_normed: w_post length")
+    if w_next is not None:
+        _dev(w_next, "w_next", torch.float32)
+        _dev(out, "out")
+        _need(w_next.numel() == width and tuple(out.shape) == (n, width) and out.dtype in DT, "add_normed: w_next / out")
+    rc = lib.add_normed(_ptr(h), _c_int(ldh), _ptr(y), _c_int(ldy), _ptr(w_post), _c_float(mult), _c_float(eps),
+                        _ptr(w_next), _ptr(out if w_next is not None else None), _c_int(n), _c_int(width),
+                        _c_int(DT[out.dtype] if w_next is not None else 0), _stream())
+    build.check(lib, rc, "add_normed")
+    return h
+
+
+def scaled_pair_sum(y, a, ya, b, yb, accumulate=False):
+    """``y = a * ya + b * yb`` (``+= `` with ``accumulate``) on float32 rows of one shape."""
+    lib = build.load("sandwich_block")
+    for name, t in (("y", y), ("ya", ya), ("yb", yb)):
+        _dev(t, name, torch.float32)
+        _need(t.shape == y.shape, "scaled_pair_sum: shapes differ")
+    rc = lib.scaled_pair_sum(_ptr(y), _c_float(a), _ptr(ya), _c_float(b), _ptr(yb), ctypes.c_long(y.numel()),
+                             _c_int(int(bool(accumulate))), _stream())
+    build.check(lib, rc, "scaled_pair_sum")
+    return y
+
+
+def head_rmsnorm(x, n_heads, head_stride, dim, weight, eps):
+    """RMS norm of the first ``dim`` columns of each of ``n_heads`` heads, ``head_stride`` columns
+    apart, of every row of ``x``, in place (csrc/head_norm.hip)."""
+    lib = build.load("head_norm")
+    ld = _rows2d(x, "x")
+    _need(x.dtype in DT, "head_rmsnorm: float32 or bfloat16")
+    _need(0 < dim <= head_stride and (n_heads - 1) * head_stride + dim <= x.shape[1], "head_rmsnorm: heads do not fit the rows")
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
+        _need(weight.numel() == dim, "head_rmsnorm: weight length")
+    rc = lib.head_rmsnorm(_ptr(x), _c_int(ld), _c_int(x.shape[0]), _c_int(n_heads), _c_int(head_stride), _c_int(dim),
+                          _ptr(weight), _c_float(eps), _c_int(DT[x.dtype]), _stream())
+    build.check(lib, rc, "head_rmsnorm")
+    return x
+
+
+# ---------------------------------------------------------------------------
+# mixers with a decaying matrix state per head (csrc/linear_state.hip)
+
+
+class ScanArgs(ctypes.Structure):
+    """Mirror of ``ScanArgs`` in csrc/linear_state.hip."""
+
+    _fields_ = [("q", _vp), ("k", _vp), ("v", _vp), ("ldq", _c_int), ("ldk", _c_int), ("ldv", _c_int),
+                ("log_a", _vp), ("decay", _vp), ("k_scale", _vp), ("k_mult", _c_float), ("skip", _vp),
+                ("rot_dims", _c_int), ("inv_freq", _vp), ("positions", _vp), ("unit_rms", _c_int), ("eps", _c_float),
+                ("gate", _vp), ("ldg", _c_int), ("out", _vp), ("ldo", _c_int), ("out_dtype", _c_int),
+                ("state", _vp), ("state_stride", _c_size_t), ("state_offset", _c_size_t), ("seq_start", _vp),
+                ("seq_len", _vp), ("slot_ids", _vp), ("n_requests", _c_int), ("H", _c_int), ("Hk", _c_int),
+                ("N", _c_int), ("P", _c_int)]
+
+
+def _f32_rows(t, name, min_cols):
+    ld = _rows2d(t, name)
+    _need(t.dtype == torch.float32, f"{name} must be float32")
+    _need(t.shape[1] >= min_cols, f"{name}: rows of {t.shape[1]} columns, {min_cols} needed")
+    return ld
+
+
+def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, n_requests, n_heads, n_key_heads,
+               key_dim, value_dim, log_a=None, decay=None, k_scale=None, k_mult=1.0, skip=None, rot_dims=0,
+               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None):
+    """``S = a S + k v^T; o = S^T q`` token by token for every (request, head), from and into the
+    requests' rows of ``state`` (float32 ``[slots, floats a request]``, head ``h``'s matrix
+    ``[key_dim, value_dim]`` at ``state_offset + h * key_dim * value_dim``).  ``q``, ``k``
+    (``[tokens, >= n_key_heads * key_dim]``), ``v`` (``[tokens, >= n_heads * value_dim]``) and
+    ``gate`` are float32 rows (column views of a projection's output are fine); ``out`` is
+    ``[tokens, n_heads * value_dim]`` in float32 or bfloat16.  See csrc/linear_state.hip for the
+    options."""
+    lib = build.load("linear_state")
+    a = ScanArgs()
+    T = out.shape[0]
+    a.ldq, a.ldk = _f32_rows(q, "q", n_key_heads * key_dim), _f32_rows(k, "k", n_key_heads * key_dim)
+    a.ldv = _f32_rows(v, "v", n_heads * value_dim)
+    _need(q.shape[0] >= T and k.shape[0] >= T and v.shape[0] >= T, "state_scan: fewer operand rows than output rows")
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    for name, t in (("log_a", log_a), ("k_scale", k_scale)):
+        if t is not None:
+            _dev(t, name, torch.float32)
+            _need(t.numel() >= T * n_heads, f"state_scan: {name} is [tokens, heads]")
+            setattr(a, name, t.data_ptr())
+    for name, t in (("decay", decay), ("skip", skip)):
+        if t is not None:
+            _dev(t, name, torch.float32)
+            _need(t.numel() == n_heads, f"state_scan: {name} has one value a head")
+            setattr(a, name, t.data_ptr())
+    _need(log_a is not None or decay is not None, "state_scan: a decay per token or per head is needed")
+    a.k_mult = float(k_mult)
+    if rot_dims:
+        _dev(inv_freq, "inv_freq", torch.float32)
+        _dev(positions, "positions", torch.int32)
+        _need(inv_freq.numel() == rot_dims // 2 and positions.numel() >= T, "state_scan: inv_freq / positions")
+        a.rot_dims, a.inv_freq, a.positions = int(rot_dims), inv_freq.data_ptr(), positions.data_ptr()
+    a.unit_rms, a.eps = int(bool(unit_rms)), float(eps)
+    if gate is not None:
+        a.ldg, a.gate = _f32_rows(gate, "gate", n_heads * value_dim), gate.data_ptr()
+    a.ldo = _rows2d(out, "out")
+    _need(out.dtype in DT and out.shape[1] == n_heads * value_dim, "state_scan: out is [tokens, heads * value_dim]")
+    a.out, a.out_dtype = out.data_ptr(), DT[out.dtype]
+    _dev(state, "state", torch.float32)
+    _need(state.dim() == 2 and state_offset + n_heads * key_dim * value_dim <= state.shape[1], "state_scan: the state rows are too short")
+    a.state, a.state_stride, a.state_offset = state.data_ptr(), state.stride(0), int(state_offset)
+    for name, t in (("seq_start", seq_start), ("seq_len", seq_len), ("slot_ids", slot_ids)):
+        _dev(t, name, torch.int32)
+        _need(t.numel() >= n_requests, f"state_scan: {name} is shorter than the requests")
+        setattr(a, name, t.data_ptr())
+    a.n_requests, a.H, a.Hk, a.N, a.P = int(n_requests), int(n_heads), int(n_key_heads), int(key_dim), int(value_dim)
+    rc = lib.state_scan(ctypes.byref(a), _stream())
+    build.check(lib, rc, "state_scan")
+    return out
+
+
+def ssm_prepare(xbc, dt, log_a, u, conv_col, dt_col, conv_w, conv_b, dt_bias, a_log, state, conv_offset, token_req,
+                seq_start, slot_ids):
+    """The causal convolution (with the requests' last inputs from ``state``), bias and silu of
+    columns ``conv_col ..`` of the float32 rows ``u`` into ``xbc``; ``dt = softplus(u[:, dt_col + h]
+    + dt_bias[h])`` and ``log_a = -exp(a_log[h]) * dt`` (csrc/linear_state.hip)."""
+    lib = build.load("linear_state")
+    ldu = _f32_rows(u, "u", 1)
+    T, C = xbc.shape
+    H = dt.shape[1]
+    taps = conv_w.shape[1]
+    for name, t in (("xbc", xbc), ("dt", dt), ("log_a", log_a), ("conv_w", conv_w), ("dt_bias", dt_bias),
+                    ("a_log", a_log), ("state", state)):
+        _dev(t, name, torch.float32)
+    if conv_b is not None:
+        _dev(conv_b, "conv_b", torch.float32)
+        _need(conv_b.numel() == C, "ssm_prepare: conv_b length")
+    _need(tuple(conv_w.shape) == (C, taps) and dt.shape == log_a.shape and dt.shape[0] == T, "ssm_prepare: shapes")
+    _need(dt_bias.numel() == H and a_log.numel() == H and u.shape[0] >= T, "ssm_prepare: per-head vectors")
+    _need(conv_col + C <= u.shape[1] and dt_col + H <= u.shape[1], "ssm_prepare: columns beyond the rows")
+    _need(state.dim() == 2 and conv_offset + (taps - 1) * C <= state.shape[1], "ssm_prepare: the state rows are too short")
+    for name, t in (("token_req", token_req), ("seq_start", seq_start), ("slot_ids", slot_ids)):
+        _dev(t, name, torch.int32)
+    rc = lib.ssm_prepare(_ptr(u), _c_int(ldu), _c_int(conv_col), _c_int(dt_col), _ptr(conv_w), _ptr(conv_b),
+                         _c_int(taps), _c_int(C), _c_int(H), _ptr(dt_bias), _ptr(a_log), _ptr(state),
+                         _c_size_t(state.stride(0)), _c_size_t(conv_offset), _ptr(token_req), _ptr(seq_start),
+                         _ptr(slot_ids), _ptr(xbc), _ptr(dt), _ptr(log_a), _c_int(T), _stream())
+    build.check(lib, rc, "ssm_prepare")
+
+
+def conv_state_update(u, conv_col, taps, n_channels, state, conv_offset, seq_start, seq_len, slot_ids, n_requests):
+    """Each request's last ``taps - 1`` inputs (columns ``conv_col ..`` of ``u``) into its state row."""
+    lib = build.load("linear_state")
+    ldu = _f32_rows(u, "u", conv_col + n_channels)
+    _dev(state, "state", torch.float32)
+    _need(state.dim() == 2 and conv_offset + (taps - 1) * n_channels <= state.shape[1], "conv_state_update: the state rows are too short")
+    for name, t in (("seq_start", seq_start), ("seq_len", seq_len), ("slot_ids", slot_ids)):
+        _dev(t, name, torch.int32)
+        _need(t.numel() >= n_requests, f"conv_state_update: {name} is shorter than the requests")
+    rc = lib.conv_state_update(_ptr(u), _c_int(ldu), _c_int(conv_col), _c_int(taps), _c_int(n_channels), _ptr(state),
+                               _c_size_t(state.stride(0)), _c_size_t(conv_offset), _ptr(seq_start), _ptr(seq_len),
+                               _ptr(slot_ids), _c_int(n_requests), _stream())
+    build.check(lib, rc, "conv_state_update")
+
+
+def gated_group_rmsnorm(out, y, z, weight, groups, eps):
+    """``out = RMSnorm(y * silu(z))`` in ``groups`` equal parts of a row, times ``weight``."""
+    lib = build.load("linear_state")
+    T, width = out.shape
+    ldy, ldz, ldo = _f32_rows(y, "y", width), _f32_rows(z, "z", width), _rows2d(out, "out")
+    _dev(weight, "weight", torch.float32)
+    _need(weight.numel() == width and out.dtype in DT and y.shape[0] >= T and z.shape[0] >= T, "gated_group_rmsnorm: shapes")
+    rc = lib.gated_group_rmsnorm(_ptr(y), _c_int(ldy), _ptr(z), _c_int(ldz), _ptr(weight), _c_float(eps), _c_int(T),
+                                 _c_int(width), _c_int(groups), _ptr(out), _c_int(ldo), _c_int(DT[out.dtype]), _stream())
+    build.check(lib, rc, "gated_group_rmsnorm")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# experts chosen per token (csrc/experts.hip)
+
+
+def router_choice(idx, weight, z, correction, top):
+    """From float32 router outputs ``z`` ``[tokens, outputs]``: softmax, the ``top`` largest of
+    softmax + ``correction`` into ``idx`` (int32 ``[tokens, top]``), their softmax values into ``weight``."""
+    lib = build.load("experts")
+    ldz = _f32_rows(z, "z", 1)
+    T, n_out = z.shape
+    _dev(idx, "idx", torch.int32)
+    _dev(weight, "weight", torch.float32)
+    _need(idx.numel() >= T * top and weight.numel() >= T * top, "router_choice: idx / weight too short")
+    if correction is not None:
+        _dev(correction, "correction", torch.float32)
+        _need(correction.numel() == n_out, "router_choice: correction length")
+    rc = lib.router_choice(_ptr(z), _c_int(ldz), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _ptr(idx),
+                           _ptr(weight), _stream())
+    build.check(lib, rc, "router_choice")
+
+
+def silu_mul(out, gate_up):
+    """``out = silu(gate_up[:, :F]) * gate_up[:, F:2F]`` with ``F = out.shape[1]``."""
+    lib = build.load("experts")
+    ld, ldo = _rows2d(gate_up, "gate_up"), _rows2d(out, "out")
+    T, F = out.shape
+    _need(gate_up.dtype == out.dtype and out.dtype in DT and gate_up.shape[1] == 2 * F and gate_up.shape[0] >= T, "silu_mul: shapes")
+    rc = lib.silu_mul(_ptr(gate_up), _c_int(ld), _ptr(out), _c_int(ldo), _c_int(T), _c_int(F), _c_int(DT[out.dtype]), _stream())
+    build.check(lib, rc, "silu_mul")
+    return out
+
+
+def expert_rows(y, x, w_gate, w_up, w_down, idx, weight, top, act, accumulate=True):
+    """``y (+)= sum over a token's picks of weight * expert(x)``, reading only the picked experts'
+    weights (``w_gate``, ``w_up``: ``[experts, F, width]``, ``w_down``: ``[experts, width, F]``); a
+    pick at or beyond the number of experts gives ``weight * x``.  ``act``: room for ``[tokens *
+    top, F]`` of ``x``'s dtype."""
+    lib = build.load("experts")
+    ldx, ldy = _rows2d(x, "x"), _rows2d(y, "y")
+    T, width = x.shape
+    n_experts = 0 if w_gate is None else w_gate.shape[0]
+    F = 1 if w_gate is None else w_gate.shape[1]
+    _need(y.dtype == torch.float32 and tuple(y.shape) == (T, width) and x.dtype in DT, "expert_rows: x / y")
+    if n_experts:
+        for name, t, shape in (("w_gate", w_gate, (n_experts, F, width)), ("w_up", w_up, (n_experts, F, width)),
+                               ("w_down", w_down, (n_experts, width, F))):
+            _dev(t, name, x.dtype)
+            _need(tuple(t.shape) == shape, f"expert_rows: {name} is {tuple(t.shape)}, want {shape}")
+        _dev(act, "act", x.dtype)
+        _need(act.numel() >= T * top * F, "expert_rows: act too small")
+    _dev(idx, "idx", torch.int32)
+    _dev(weight, "weight", torch.float32)
+    _need(idx.numel() >= T * top and weight.numel() >= T * top, "expert_rows: idx / weight too short")
+    rc = lib.expert_rows(_ptr(x), _c_int(ldx), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(idx), _ptr(weight),
+                         _c_int(T), _c_int(n_experts), _c_int(top), _c_int(F), _c_int(width), _ptr(act), _ptr(y),
+                         _c_int(ldy), _c_int(int(bool(accumulate))), _c_int(DT[x.dtype]), _stream())
+    build.check(lib, rc, "expert_rows")
+    return y

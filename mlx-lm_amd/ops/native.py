@@ -82,7 +82,7 @@ class EngCtx(Structure):
 class EngCall(Structure):
     _fields_ = [("x", EngMat), ("residual", EngMat), ("out", EngMat), ("q", EngMat), ("k", EngMat),
                 ("rows", c_void_p), ("n_rows", c_int), ("cache_slot", c_int), ("writes_cache", c_int),
-                ("lazy", c_int), ("result", EngMat), ("index", c_void_p), ("nbytes", c_size_t)]
+                ("lazy", c_int), ("state_slot", c_int), ("pad_", c_int), ("result", EngMat), ("index", c_void_p), ("nbytes", c_size_t)]
 
 
 class EngScatter(Structure):
@@ -301,7 +301,11 @@ def run_python_part(part, method, ctx, call):
     elif method == CB_FFN:
         part.forward(ctx, T(call.x), T(call.residual))
     elif method == CB_BLOCK:
-        part.forward(ctx, T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
+        if call.state_slot >= 0:
+            part.forward(ctx, T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache),
+                         state=ctx.cache_view(call.state_slot))
+        else:
+            part.forward(ctx, T(call.residual), ctx.cache_view(call.cache_slot), bool(call.writes_cache))
     elif method == CB_NORM:
         x = T(call.x)
         if call.rows:

@@ -1,6 +1,7 @@
 """Parts that models are put together from; importing this registers the built-in kinds."""
 
-from . import attention, block, embedding, feed_forward, gated_attention, head, norms, positions  # noqa: F401
+from . import (attention, block, embedding, experts, feed_forward, gated_attention, head, linear_state, norms,  # noqa: F401
+               positions)
 from .base import (
     BLOCKS,
     EMBEDDINGS,

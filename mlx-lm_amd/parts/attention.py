@@ -2,6 +2,8 @@
 
 import ctypes
 
+import torch
+
 from ..config.plan import CacheNeed
 from ..ops import kernels, native
 from .base import POSITION_ENCODINGS, Mixer, TensorSpec, build_part, register_mixer, value_of
@@ -24,11 +26,18 @@ class CausalSelfAttention(Mixer):
     shares each key head among a group of query heads; ``window`` limits a
     query to the last ``window`` keys; ``position`` may rotate queries and keys
     before the cache write.
+
+    ``split_names = (q, k, v, o)``: the checkpoint holds the four matrices apart (no biases), with
+    keys of ``key_dim`` and values of ``value_dim`` columns a head.  They are laid into the fused
+    layout with every head padded by zero rows (``o``: zero columns) to ``head_dim``, which the
+    kernels and the cache then see: a padded key column adds nothing to a score, a padded value
+    column meets a zero column of ``o``.
     """
 
 
     def __init__(self, width, n_heads, head_dim, n_kv_heads=None, scale=None, bias=True, window=0,
-                 position=None, qkv_name="c_attn", out_name="c_proj", prefix=""):
+                 position=None, qkv_name="c_attn", out_name="c_proj", split_names=None, key_dim=None,
+                 value_dim=None, prefix=""):
         super().__init__(prefix)
         n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads:
@@ -45,6 +54,13 @@ class CausalSelfAttention(Mixer):
         self.q_width = n_heads * head_dim
         self.kv_width = n_kv_heads * head_dim
         self.qkv_name, self.out_name = qkv_name, out_name
+        self.split_names = tuple(split_names) if split_names is not None else None
+        self.key_dim, self.value_dim = int(key_dim or head_dim), int(value_dim or head_dim)
+        if self.split_names is None and (self.key_dim, self.value_dim) != (head_dim, head_dim):
+            raise ValueError("keys and values narrower than head_dim come as separate tensors (split_names)")
+        if self.split_names is not None and (bias or len(self.split_names) != 4
+                                             or not 0 < self.key_dim <= head_dim or not 0 < self.value_dim <= head_dim):
+            raise ValueError("split_names: four names (q, k, v, o), no biases, key_dim and value_dim within head_dim")
         self.position = (
             build_part(POSITION_ENCODINGS, "position encoding", position) if position is not None else None
         )
@@ -58,6 +74,15 @@ class CausalSelfAttention(Mixer):
 
     def tensors(self):
         n = self._name
+        if self.split_names is not None:
+            q, k, v, o = (n(x) for x in self.split_names)
+            t = {q: TensorSpec((self.n_heads * self.key_dim, self.width), "matrix"),
+                 k: TensorSpec((self.n_kv_heads * self.key_dim, self.width), "matrix"),
+                 v: TensorSpec((self.n_kv_heads * self.value_dim, self.width), "matrix"),
+                 o: TensorSpec((self.width, self.n_heads * self.value_dim), "matrix")}
+            if self.position is not None:
+                t.update(self.position.tensors())
+            return t
         t = {
             n(self.qkv_name + ".weight"): TensorSpec((self.q_width + 2 * self.kv_width, self.width), "matrix"),
             n(self.out_name + ".weight"): TensorSpec((self.width, self.q_width), "matrix"),
@@ -69,10 +94,24 @@ class CausalSelfAttention(Mixer):
             t.update(self.position.tensors())
         return t
 
+    def _padded_heads(self, w, n_heads, dim):
+        """``[n_heads * dim, width]`` with every head's rows padded by zeros to ``head_dim``."""
+        w = w.view(n_heads, dim, self.width)
+        return torch.cat([w, w.new_zeros(n_heads, self.head_dim - dim, self.width)], 1).reshape(-1, self.width)
+
     def load(self, tensors):
         n = self._name
-        self.qkv_w = tensors[n(self.qkv_name + ".weight")]
-        self.out_w = tensors[n(self.out_name + ".weight")]
+        if self.split_names is not None:
+            q, k, v, o = (tensors[n(x)] for x in self.split_names)
+            self.qkv_w = torch.cat([self._padded_heads(q, self.n_heads, self.key_dim),
+                                    self._padded_heads(k, self.n_kv_heads, self.key_dim),
+                                    self._padded_heads(v, self.n_kv_heads, self.value_dim)]).contiguous()
+            o = o.view(self.width, self.n_heads, self.value_dim)
+            self.out_w = torch.cat([o, o.new_zeros(self.width, self.n_heads, self.head_dim - self.value_dim)],
+                                   2).reshape(self.width, -1).contiguous()
+        else:
+            self.qkv_w = tensors[n(self.qkv_name + ".weight")]
+            self.out_w = tensors[n(self.out_name + ".weight")]
         if self.has_bias:
             self.qkv_b = tensors[n(self.qkv_name + ".bias")]
             self.out_b = tensors[n(self.out_name + ".bias")]

@@ -126,5 +126,90 @@ class PostNormBlock(Block):
         return h
 
 
+class SandwichBlock(Block):
+    """``h += m * post1(mixer(pre1(h))); h += m * post2(ffn(pre2(h)))``: every sublayer has a norm
+    ahead of it and one behind it, and its normed output enters the stream times ``residual_mult``.
+
+    The four norms are LayerNorms with a weight and no bias (``layernorm`` parts give weight and
+    eps).  The sublayers write their outputs as float32 rows (a part that can only add gets rows
+    of zeros); the norm behind a sublayer, the scaled sum into the float32 stream and the norm
+    ahead of the next sublayer are one kernel (csrc/sandwich_block.hip).  The feed-forward, with
+    its two norms, may be absent.  A mixer that keeps pages and per-request state at once
+    (``wants_state``) gets the run's state slot beside its cache slot.  No counterpart in
+    mlx_lm/models/gpt2.py, whose blocks norm ahead of their sublayers only (:98-108).
+    """
+
+    PARTS = {"mixer_norm": "norm", "mixer": "mixer", "mixer_post_norm": "norm", "ffn_norm": "norm",
+             "ffn": "feed_forward", "ffn_post_norm": "norm"}
+    OPTIONAL = ("ffn_norm", "ffn", "ffn_post_norm")
+
+    def __init__(self, mixer_norm, mixer, mixer_post_norm, ffn_norm=None, ffn=None, ffn_post_norm=None,
+                 residual_mult=1.0, prefix=""):
+        super().__init__(prefix)
+        if len({ffn is None, ffn_norm is None, ffn_post_norm is None}) != 1:
+            raise ValueError("a layer has a feed-forward and its two norms, or none of the three")
+        norms = [n for n in (mixer_norm, mixer_post_norm, ffn_norm, ffn_post_norm) if n is not None]
+        for n in norms:
+            if not (hasattr(n, "weight") and hasattr(n, "eps")) or getattr(n, "has_bias", True):
+                raise ValueError(f"this arrangement fuses LayerNorms without a bias, not a {type(n).__name__}")
+            if n.eps != norms[0].eps or n.width != norms[0].width:
+                raise ValueError("the norms of a layer share width and eps")
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ffn_norm, self.ffn, self.ffn_post_norm = ffn_norm, ffn, ffn_post_norm
+        self.width, self.eps, self.residual_mult = norms[0].width, norms[0].eps, float(residual_mult)
+        for part in (mixer, ffn):
+            if part is not None and getattr(part, "can_overwrite", False) and hasattr(part, "overwrite"):
+                part.overwrite = True
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.parts())
+
+    def parts(self):
+        out = []
+
+        def walk(part):
+            if part is None:
+                return
+            out.append(part)
+            for sub in getattr(part, "sub_parts", lambda: ())():
+                walk(sub)
+
+        for p in (self.mixer_norm, self.mixer, self.mixer_post_norm, self.ffn_norm, self.ffn, self.ffn_post_norm):
+            walk(p)
+        return tuple(out)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def state_need(self):
+        return self.mixer.state_need() if hasattr(self.mixer, "state_need") else None
+
+    def forward(self, ctx, h, cache, writes_cache=True, state=None):
+        import torch
+
+        from ..ops import kernels
+
+        T = h.shape[0]
+        mark = ctx.scratch_mark()
+        x = ctx.scratch((T, self.width), ctx.dtype)
+        kernels.layernorm(x, h, self.mixer_norm.weight, None, self.eps)
+        y = ctx.scratch((T, self.width), torch.float32)
+        if not getattr(self.mixer, "overwrite", False):
+            y.zero_()
+        if getattr(self.mixer, "wants_state", False):
+            self.mixer.forward(ctx, x, y, cache, writes_cache, state=state)
+        else:
+            self.mixer.forward(ctx, x, y, cache, writes_cache)
+        if self.ffn is None:
+            kernels.add_normed(h, y, self.mixer_post_norm.weight, self.residual_mult, self.eps)
+        else:
+            kernels.add_normed(h, y, self.mixer_post_norm.weight, self.residual_mult, self.eps, self.ffn_norm.weight, x)
+            if not getattr(self.ffn, "overwrite", False):
+                y.zero_()
+            self.ffn.forward(ctx, x, y)
+            kernels.add_normed(h, y, self.ffn_post_norm.weight, self.residual_mult, self.eps)
+        ctx.scratch_release(mark)
+        return h
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("sandwich", SandwichBlock)
 register_block("post_norm", PostNormBlock)

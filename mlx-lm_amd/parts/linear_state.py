@@ -1,0 +1,241 @@
+"""Mixers whose memory of a sequence is a decaying matrix per head, kept per request between steps."""
+
+import torch
+
+from ..config.plan import StateNeed
+from ..ops import kernels
+from .base import Mixer, TensorSpec, register_mixer
+
+
+class _SequenceArrays:
+    """The step arrays that a scan over each request's own tokens needs: where a request's tokens
+    start in the flat batch and how many they are (its state row is ``ctx.slot_ids``)."""
+
+    step_arrays_key = "sequences"
+    step_array_names = ("starts", "lens")
+
+    @staticmethod
+    def step_arrays(batch):
+        return {"starts": list(batch.q_starts), "lens": list(batch.q_lens)}
+
+
+def _matrix(w):
+    return kernels.for_decode(w.contiguous())
+
+
+class Retention(_SequenceArrays, Mixer):
+    """Linear attention with a fixed decay per head and neither softmax nor denominator:
+
+        ``S_t = decay_h S_(t-1) + k_t v_t^T``,   ``o_t = S_t^T q_t``
+
+    with ``q = Wq x``, ``k = Wk x`` (``n_heads x key_dim``), ``v = Wv x`` (``n_heads x value_dim``).
+    Queries and keys turn with the position on their first ``rot_dims`` columns (column ``i`` with
+    column ``i + rot_dims / 2`` by ``position * rot_base^(-2i / rot_dims)``); keys are then
+    multiplied by ``key_dim^(-1/2)`` (``key_scale``).  Each head's ``o`` is divided by its root
+    mean square (``eps``), the heads are multiplied by ``silu(Wg x)`` and projected by ``Wo``.
+    ``S`` (``key_dim x value_dim`` a head, float32, zero at a request's start) is the request's
+    state.  One product gives ``[q | k | v | g]`` as float32 rows; angles, the recurrence, the
+    norm and the gate are 32-bit (csrc/linear_state.hip).  No counterpart in
+    mlx_lm/models/gpt2.py.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    can_overwrite = True  # writes its output instead of adding it where ``overwrite`` is set
+
+    def __init__(self, width, n_heads, key_dim, value_dim, decay, eps, rot_dims=0, rot_base=10000.0, key_scale=None,
+                 names=("q", "k", "v", "g", "o"), prefix=""):
+        super().__init__(prefix)
+        if n_heads <= 0 or key_dim <= 0 or not 0 < value_dim <= 256:
+            raise ValueError(f"{n_heads} heads of keys {key_dim} and values {value_dim} (values at most 256)")
+        if len(decay) != n_heads:
+            raise ValueError(f"{len(decay)} decays for {n_heads} heads")
+        if rot_dims % 2 or not 0 <= rot_dims <= key_dim:
+            raise ValueError(f"{rot_dims} turning columns of {key_dim}: an even number within the head")
+        if width % 8 or (n_heads * value_dim) % 8:
+            raise ValueError(f"width {width} and the heads' value columns {n_heads * value_dim} must be multiples of 8")
+        self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
+        self.decay_values, self.eps = [float(d) for d in decay], float(eps)
+        self.rot_dims, self.rot_base = int(rot_dims), float(rot_base)
+        self.key_scale = float(key_scale) if key_scale is not None else key_dim**-0.5
+        self.qk_width, self.v_width = n_heads * key_dim, n_heads * value_dim
+        self.names = dict(zip(("q", "k", "v", "g", "o"), (self._name(n) for n in names)))
+        self.overwrite = False
+        self.in_w = self.out_w = self.decay = self.inv_freq = None
+
+    def cache_need(self):
+        return StateNeed((self.n_heads * self.key_dim * self.value_dim,), "float32")
+
+    def tensors(self):
+        n = self.names
+        return {n["q"]: TensorSpec((self.qk_width, self.width), "matrix"),
+                n["k"]: TensorSpec((self.qk_width, self.width), "matrix"),
+                n["v"]: TensorSpec((self.v_width, self.width), "matrix"),
+                n["g"]: TensorSpec((self.v_width, self.width), "matrix"),
+                n["o"]: TensorSpec((self.width, self.v_width), "matrix")}
+
+    def load(self, tensors):
+        n = self.names
+        dev = tensors[n["q"]].device
+        self.in_w = _matrix(torch.cat([tensors[n[x]] for x in ("q", "k", "v", "g")]))
+        self.out_w = _matrix(tensors[n["o"]])
+        self.first_weight = self.in_w
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=dev)
+        half = self.rot_dims // 2
+        if half:
+            i = torch.arange(half, dtype=torch.float64)
+            self.inv_freq = torch.pow(torch.tensor(self.rot_base, dtype=torch.float64), -2.0 * i / self.rot_dims).float().to(dev)
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        T = x.shape[0]
+        mark = ctx.scratch_mark()
+        u = ctx.scratch((T, 2 * self.qk_width + 2 * self.v_width), torch.float32)
+        kernels.linear(u, x, self.in_w)
+        a, b = self.qk_width, 2 * self.qk_width
+        out = ctx.scratch((T, self.v_width), ctx.dtype)
+        kernels.state_scan(out, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, 0,
+                           ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
+                           self.n_heads, self.n_heads, self.key_dim, self.value_dim, decay=self.decay,
+                           k_mult=self.key_scale, rot_dims=self.rot_dims, inv_freq=self.inv_freq,
+                           positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:])
+        kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
+        ctx.scratch_release(mark)
+
+
+class StateSpace(_SequenceArrays, Mixer):
+    """The selective state space with a scalar decay a head:
+
+        ``S_t = exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T``,   ``y_t = S_t^T C_t + D_h x_t``
+
+    ``Win x`` is laid out ``[z: inner | x: inner | B: groups * state | C: groups * state | dt: heads]``
+    with ``inner = n_heads * value_dim``; ``x``, ``B`` and ``C`` pass a causal convolution per
+    channel (``taps`` taps, the last for the current token, zeros before a request's start, a
+    bias) and a silu; ``dt = softplus(dt + dt_bias)``; head ``h`` reads group ``h // (n_heads /
+    groups)``.  ``y * silu(z)`` is RMS-normed in ``norm_groups`` equal parts, multiplied by a
+    weight and projected by ``Wo``.  A request's state is its last ``taps - 1`` convolution inputs
+    and ``S`` (``state x value_dim`` a head), float32, zero at its start.  The projection writes
+    float32 rows; everything up to the normed output is 32-bit (csrc/linear_state.hip).  No
+    counterpart in mlx_lm/models/gpt2.py.
+    """
+
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, width, n_heads, value_dim, state, groups, taps, norm_groups, eps,
+                 names=("in", "conv", "conv.b", "dt_bias", "A_log", "D", "norm", "o"), prefix=""):
+        super().__init__(prefix)
+        if n_heads <= 0 or groups <= 0 or n_heads % groups:
+            raise ValueError(f"{n_heads} heads cannot be grouped over {groups} groups")
+        if not 0 < value_dim <= 256 or state <= 0 or taps < 1:
+            raise ValueError(f"values of {value_dim} (at most 256), a state of {state}, {taps} taps")
+        inner = n_heads * value_dim
+        if norm_groups <= 0 or inner % norm_groups:
+            raise ValueError(f"{inner} inner columns cannot be normed in {norm_groups} equal parts")
+        if width % 8 or inner % 8:
+            raise ValueError(f"width {width} and the inner size {inner} must be multiples of 8")
+        self.width, self.n_heads, self.value_dim, self.state, self.groups = width, n_heads, value_dim, state, groups
+        self.taps, self.norm_groups, self.eps, self.inner = int(taps), int(norm_groups), float(eps), inner
+        self.channels = inner + 2 * groups * state
+        self.in_width = 2 * inner + 2 * groups * state + n_heads
+        keys = ("in", "conv", "conv.b", "dt_bias", "A_log", "D", "norm", "o")
+        self.names = dict(zip(keys, (self._name(n) for n in names)))
+        self.conv_floats = (self.taps - 1) * self.channels
+        self.overwrite = False
+
+    def cache_need(self):
+        return StateNeed((self.conv_floats + self.n_heads * self.state * self.value_dim,), "float32")
+
+    def tensors(self):
+        n = self.names
+        return {n["in"]: TensorSpec((self.in_width, self.width), "matrix"),
+                n["conv"]: TensorSpec((self.channels, self.taps), "vector"),
+                n["conv.b"]: TensorSpec((self.channels,), "vector"),
+                n["dt_bias"]: TensorSpec((self.n_heads,), "vector"),
+                n["A_log"]: TensorSpec((self.n_heads,), "vector"),
+                n["D"]: TensorSpec((self.n_heads,), "vector"),
+                n["norm"]: TensorSpec((self.inner,), "vector"),
+                n["o"]: TensorSpec((self.width, self.inner), "matrix")}
+
+    def load(self, tensors):
+        n = self.names
+        self.in_w, self.out_w = _matrix(tensors[n["in"]]), _matrix(tensors[n["o"]])
+        self.first_weight = self.in_w
+        self.conv_w, self.conv_b = tensors[n["conv"]].contiguous(), tensors[n["conv.b"]]
+        self.dt_bias, self.a_log, self.skip = tensors[n["dt_bias"]], tensors[n["A_log"]], tensors[n["D"]]
+        self.norm_w = tensors[n["norm"]]
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        T, H, GN = x.shape[0], self.n_heads, self.groups * self.state
+        mark = ctx.scratch_mark()
+        u = ctx.scratch((T, self.in_width), torch.float32)
+        kernels.linear(u, x, self.in_w)
+        xbc = ctx.scratch((T, self.channels), torch.float32)
+        dt = ctx.scratch((T, H), torch.float32)
+        log_a = ctx.scratch((T, H), torch.float32)
+        starts, lens = ctx.array("sequences.starts"), ctx.array("sequences.lens")
+        kernels.ssm_prepare(xbc, dt, log_a, u, self.inner, self.inner + self.channels, self.conv_w, self.conv_b,
+                            self.dt_bias, self.a_log, cache.state, 0, ctx.token_req, starts, ctx.slot_ids)
+        kernels.conv_state_update(u, self.inner, self.taps, self.channels, cache.state, 0, starts, lens, ctx.slot_ids,
+                                  ctx.n_requests)
+        y = ctx.scratch((T, self.inner), torch.float32)
+        kernels.state_scan(y, xbc[:, self.inner + GN:], xbc[:, self.inner:self.inner + GN], xbc[:, :self.inner],
+                           cache.state, self.conv_floats, starts, lens, ctx.slot_ids, ctx.n_requests, H, self.groups,
+                           self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip)
+        out = ctx.scratch((T, self.inner), ctx.dtype)
+        kernels.gated_group_rmsnorm(out, y, u[:, :self.inner], self.norm_w, self.norm_groups, self.eps)
+        kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
+        ctx.scratch_release(mark)
+
+
+class ParallelMixers(Mixer):
+    """Two mixers side by side that read the same input: ``left_scale * left(x) + right_scale *
+    right(x)``.  The left one keeps the run's cache slot, the right one the run's state slot (the
+    arrangement passes both on: ``wants_state``).  The two outputs are float32 rows and are summed
+    in float32."""
+
+    can_overwrite = True
+    wants_state = True
+
+    def __init__(self, left, right, left_scale=1.0, right_scale=1.0, prefix=""):
+        from .base import MIXERS, build_part
+
+        super().__init__(prefix)
+        self.left = build_part(MIXERS, "mixer", left)
+        self.right = build_part(MIXERS, "mixer", right)
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self.overwrite = False
+        for m in (self.left, self.right):
+            if getattr(m, "can_overwrite", False) and hasattr(m, "overwrite"):
+                m.overwrite = True
+        self.graph_safe = all(getattr(m, "graph_safe", False) for m in (self.left, self.right))
+
+    def sub_parts(self):
+        return (self.left, self.right)
+
+    def cache_need(self):
+        return self.left.cache_need()
+
+    def state_need(self):
+        need = self.right.cache_need()
+        if need is not None and not isinstance(need, StateNeed):
+            raise ValueError("the right one of two parallel mixers keeps per-request state or nothing")
+        return need
+
+    # (the two mixers are parts of the model in their own right, ``sub_parts``: the model hands
+    # them their tensors and asks them for their step arrays; nothing here owns a tensor)
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True, state=None):
+        mark = ctx.scratch_mark()
+        outs = []
+        for m, slot in ((self.left, cache), (self.right, state)):
+            y = ctx.scratch(tuple(residual.shape), torch.float32)
+            if not getattr(m, "overwrite", False):
+                y.zero_()
+            m.forward(ctx, x, y, slot, writes_cache)
+            outs.append(y)
+        kernels.scaled_pair_sum(residual, self.left_scale, outs[0], self.right_scale, outs[1], accumulate=not self.overwrite)
+        ctx.scratch_release(mark)
+
+
+register_mixer("retention", Retention)
+register_mixer("state_space", StateSpace)
+register_mixer("parallel", ParallelMixers)

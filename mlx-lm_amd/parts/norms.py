@@ -16,20 +16,21 @@ class LayerNorm(Norm):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
 
-    def __init__(self, width, eps, bias=True, prefix=""):
+    def __init__(self, width, eps, bias=True, weight_name="weight", bias_name="bias", prefix=""):
         super().__init__(prefix)
         self.width, self.eps, self.has_bias = width, float(eps), bias
+        self.weight_name, self.bias_name = self._name(weight_name), self._name(bias_name)
         self.weight = self.bias = None
 
     def tensors(self):
-        t = {self._name("weight"): TensorSpec((self.width,), "vector")}
+        t = {self.weight_name: TensorSpec((self.width,), "vector")}
         if self.has_bias:
-            t[self._name("bias")] = TensorSpec((self.width,), "vector")
+            t[self.bias_name] = TensorSpec((self.width,), "vector")
         return t
 
     def load(self, tensors):
-        self.weight = tensors[self._name("weight")]
-        self.bias = tensors[self._name("bias")] if self.has_bias else None
+        self.weight = tensors[self.weight_name]
+        self.bias = tensors[self.bias_name] if self.has_bias else None
 
     settles_pending = True  # adds a sum that is pending on ``x`` before (or while) it norms the rows
     reads_ahead = True  # ``forward`` takes ``ahead``, the weights that its result meets first

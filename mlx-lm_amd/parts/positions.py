@@ -53,5 +53,39 @@ class LearnedPositions(PositionEncoding):
         return self.table, ctx.positions
 
 
+class HeadRMSNorm(PositionEncoding):
+    """Queries and keys divided by their root mean square over a head and multiplied by a weight
+    of ``dim`` values that all heads share (one for queries, one for keys), in place, ahead of the
+    cache write: the hook that the attention part offers for what happens to queries and keys
+    between their projection and the scores.  Positions do not enter.  Heads may lie
+    ``head_stride`` columns apart (padded beyond ``dim``).  32-bit inside (csrc/head_norm.hip).
+    No counterpart in mlx_lm/models/gpt2.py, whose attention (:44-68) norms neither.
+    """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
+    def __init__(self, dim, eps, head_stride=None, q_name="q.norm", k_name="k.norm", prefix=""):
+        super().__init__(prefix)
+        self.dim, self.eps = int(dim), float(eps)
+        self.head_stride = int(head_stride or dim)
+        if not 0 < self.dim <= self.head_stride:
+            raise ValueError(f"a head of {self.dim} columns does not fit a stride of {self.head_stride}")
+        self.q_name, self.k_name = self._name(q_name), self._name(k_name)
+        self.q_weight = self.k_weight = None
+
+    def tensors(self):
+        return {self.q_name: TensorSpec((self.dim,), "vector"), self.k_name: TensorSpec((self.dim,), "vector")}
+
+    def load(self, tensors):
+        self.q_weight, self.k_weight = tensors[self.q_name], tensors[self.k_name]
+
+    def rotate(self, ctx, q, k):
+        from ..ops import kernels
+
+        kernels.head_rmsnorm(q, q.shape[1] // self.head_stride, self.head_stride, self.dim, self.q_weight, self.eps)
+        kernels.head_rmsnorm(k, k.shape[1] // self.head_stride, self.head_stride, self.dim, self.k_weight, self.eps)
+
+
 register_position_encoding("none", NoPositions)
+register_position_encoding("head_rmsnorm", HeadRMSNorm)
 register_position_encoding("learned", LearnedPositions)
