@@ -47,7 +47,7 @@ def rotate_half(x, positions, dims, base):
 
 def retention(h, t, p, m, eps):
     """Linear attention with one fixed decay a head, no softmax: ``S = g S + k v^T; o = S^T q``."""
-    T, H, d, dv = h.shape[0], m["heads"], m["dim"], m["vdim"]
+    T, H, d, dv = h.shape[0], m["heads"], m["dim"], m.get("vdim", m["dim"])
     pos = torch.arange(T)
     q = (h @ t[p + "q"].T).view(T, H, d)
     k = (h @ t[p + "k"].T).view(T, H, d)
@@ -74,7 +74,7 @@ def window_mask(T, size):
 def window_attention(h, t, p, m, eps):
     """Softmax attention over the last ``mask.size`` tokens, grouped key heads, RMS-normed queries and
     keys with a weight shared by the heads, values of their own width, no positions."""
-    T, H, G, d, dv = h.shape[0], m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
+    T, H, G, d, dv = h.shape[0], m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
     q = unit_rms((h @ t[p + "q"].T).view(T, H, d), eps) * t[p + "q.norm"]
     k = unit_rms((h @ t[p + "k"].T).view(T, G, d), eps) * t[p + "k.norm"]
     v = (h @ t[p + "v"].T).view(T, G, dv)
@@ -82,7 +82,7 @@ def window_attention(h, t, p, m, eps):
     out = torch.zeros(T, H, dv, dtype=F64)
     for hd in range(H):
         g = hd // (H // G)
-        s = (q[:, hd] @ k[:, g].T) * m["scale"]
+        s = (q[:, hd] @ k[:, g].T) * m.get("scale", d ** -0.5)
         s = s.masked_fill(~seen, -math.inf)
         out[:, hd] = torch.softmax(s, -1) @ v[:, g]
     return out.reshape(T, H * dv) @ t[p + "o"].T
@@ -180,3 +180,55 @@ def model(tensors, cfg, tokens, streams=None):
         if streams is not None:
             streams.append(x)
     return layer_norm(x, t["final.norm"], cfg["norm"]["eps"]) @ t["head"].T
+
+
+def random_weights(cfg, seed, sharp=1.0):
+    """Float32 tensors under the checkpoint's names, every vector drawn (no ones, no zeros).
+    ``sharp`` scales the attention's query and key weights, so that its softmax is peaked and a
+    key on the wrong side of the window's edge shows."""
+    g = torch.Generator().manual_seed(seed)
+    D = cfg["width"]
+
+    def normal(shape, std, mean=0.0):
+        return torch.randn(shape, generator=g) * std + mean
+
+    t = {"embed": normal((cfg["vocab"], D), 1.0), "final.norm": normal((D,), 0.1, 1.0),
+         "head": normal((cfg["vocab"], D), D ** -0.5)}
+    for i, entry in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", entry["mixer"]
+        t[p + "norm1"], t[p + "norm1b"] = normal((D,), 0.1, 1.0), normal((D,), 0.1, 1.0)
+        if entry["type"] == "retention":
+            H, d, dv = m["heads"], m["dim"], m.get("vdim", m["dim"])
+            for name, n in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
+                t[p + "mix." + name] = normal((n, D), D ** -0.5)
+            t[p + "mix.o"] = normal((D, H * dv), (H * dv) ** -0.5)
+        else:
+            a, b = m["left"], m["right"]
+            H, G, d, dv = a["heads"], a.get("kv_heads", a["heads"]), a["dim"], a.get("vdim", a["dim"])
+            q = p + "mix.left."
+            t[q + "q"], t[q + "k"] = normal((H * d, D), D ** -0.5) * sharp, normal((G * d, D), D ** -0.5) * sharp
+            t[q + "v"], t[q + "o"] = normal((G * dv, D), D ** -0.5), normal((D, H * dv), (H * dv) ** -0.5)
+            t[q + "q.norm"], t[q + "k.norm"] = normal((d,), 0.2, 1.0) * sharp, normal((d,), 0.2, 1.0) * sharp
+            r = p + "mix.right."
+            Hs, P, N, Gs, taps = b["heads"], b["vdim"], b["state"], b["groups"], b["conv"]
+            inner, C = Hs * P, Hs * P + 2 * Gs * N
+            t[r + "in"] = normal((2 * inner + 2 * Gs * N + Hs, D), D ** -0.5)
+            t[r + "conv"], t[r + "conv.b"] = normal((C, taps), 0.5), normal((C,), 0.2)
+            t[r + "dt_bias"], t[r + "A_log"] = normal((Hs,), 0.5), normal((Hs,), 0.5, -1.5)
+            t[r + "D"], t[r + "norm"] = normal((Hs,), 0.3, 1.0), normal((inner,), 0.1, 1.0)
+            t[r + "o"] = normal((D, inner), inner ** -0.5)
+        mlp = entry.get("mlp")
+        if mlp is not None:
+            q, r = p + "mlp.", mlp["router"]
+            t[p + "norm2"], t[p + "norm2b"] = normal((D,), 0.1, 1.0), normal((D,), 0.1, 1.0)
+            F = (mlp.get("expert") or {}).get("ff", 0)
+            for e in range(r["experts"]):
+                t[f"{q}e{e}.gate"], t[f"{q}e{e}.up"] = normal((F, D), D ** -0.5), normal((F, D), D ** -0.5)
+                t[f"{q}e{e}.down"] = normal((D, F), F ** -0.5)
+            n_out = r["experts"] + r.get("identity", 0)
+            t[q + "router"], t[q + "correction"] = normal((n_out, D), 1.5 * D ** -0.5), normal((n_out,), 0.05)
+            Fs = (mlp.get("shared") or {}).get("ff", 0)
+            if Fs:
+                t[q + "shared.gate"], t[q + "shared.up"] = normal((Fs, D), D ** -0.5), normal((Fs, D), D ** -0.5)
+                t[q + "shared.down"] = normal((D, Fs), Fs ** -0.5)
+    return t
