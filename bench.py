@@ -32,7 +32,8 @@ vocabulary and positions; every Pafutar head with a key head of its own, as GPT-
 prefill of 2 x 1,024 tokens and decode at batch 1, 8 and 32 from context 512, for each of
 ``DESIGN_SIZES`` (``--design-size`` names one, ``--design-only`` one design, for a profile).  The
 Pafutar model runs once without a window (like for like with GPT-2's attention) and once with a
-window of 512 that keeps the first 64 tokens.  It prints one JSON line of its own.
+window of 512 that keeps the first 64 tokens.  Ruzolorn runs at the same layer sizes too
+(``ruzolorn_config``), without a window and with one of 512.  It prints one JSON line of its own.
 """
 
 import argparse
@@ -68,6 +69,8 @@ def design_config(design, size, window=None):
         return dict(model_type="gpt2", n_layer=s["layers"], n_embd=s["width"], n_head=s["heads"], n_inner=s["ff"],
                     vocab_size=DESIGN_VOCAB, n_positions=DESIGN_POSITIONS, layer_norm_epsilon=1e-5,
                     activation_function="gelu_new")
+    if design == "ruzolorn":
+        return ruzolorn_config(s, window)
     mixer = {"heads": s["heads"], "kv_heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5}
     if window:
         mixer["mask"] = {"size": window[0], "keep_first": window[1]}
@@ -75,6 +78,29 @@ def design_config(design, size, window=None):
     return {"architecture": "Pafutar", "vocab": DESIGN_VOCAB, "width": s["width"], "max_positions": DESIGN_POSITIONS,
             "embedding": {"scale": s["width"] ** 0.5}, "norm": {"eps": 1e-6}, "postln_alpha": 2.0,
             "layers": [dict(layer) for _ in range(s["layers"])]}
+
+
+def ruzolorn_config(s, window=None):
+    """Ruzolorn at GPT-2's layer sizes: retention layers and parallel layers by turns, as many heads
+    of the same size (a key head for every query head in the attention, as GPT-2 has; the state
+    space as wide as the model, a state as large as a head), and a feed-forward of sixteen experts
+    and two identity experts of which a token uses four, each an eighth of GPT-2's inner size, with
+    a shared expert of a quarter of it: a token multiplies with 3 x (4/8 + 1/4) = 2.25 inner sizes
+    of weights where GPT-2's does with 2."""
+    H, d, D = s["heads"], s["dim"], s["width"]
+    decay = [1.0 - 2.0 ** (-5.0 - 5.0 * h / max(1, H - 1)) for h in range(H)]
+    retention = {"type": "retention", "mixer": {"heads": H, "dim": d, "vdim": d, "decay": decay,
+                                                "rot": {"dims": d, "base": 10000.0}}}
+    left = {"heads": H, "kv_heads": H, "dim": d, "vdim": d, "scale": d ** -0.5}
+    if window:
+        left["mask"] = {"size": window[0]}
+    right = {"heads": H, "vdim": d, "state": d, "groups": 1, "conv": 4, "norm_groups": 1}
+    parallel = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}}
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"] // 8}, "router": {"experts": 16, "identity": 2, "top": 4},
+           "shared": {"ff": s["ff"] // 4}}
+    layers = [dict(retention if i % 2 == 0 else parallel, mlp=mlp) for i in range(s["layers"])]
+    return {"architecture": "Ruzolorn", "vocab": DESIGN_VOCAB, "width": D, "max_positions": DESIGN_POSITIONS,
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "residual_mult": 0.7, "layers": layers}
 
 
 def bench_design(config, dtype, batches, steps, warmup):
@@ -123,7 +149,8 @@ def compare_designs(a):
             "steps": a.steps, "warmup": a.warmup, "vocab": DESIGN_VOCAB, "positions": DESIGN_POSITIONS, "sizes": {}}
     for size in sizes:
         entry = {"layer_sizes": DESIGN_SIZES[size]}
-        runs = {"gpt2": ("gpt2", None), "pafutar": ("pafutar", None), "pafutar_window_512_keep_64": ("pafutar", (512, 64))}
+        runs = {"gpt2": ("gpt2", None), "pafutar": ("pafutar", None), "pafutar_window_512_keep_64": ("pafutar", (512, 64)),
+                "ruzolorn": ("ruzolorn", None), "ruzolorn_window_512": ("ruzolorn", (512, 0))}
         for name, (design, window) in runs.items():
             if a.design_only and name != a.design_only:
                 continue
@@ -232,7 +259,7 @@ def main():
     ap.add_argument("--designs", action="store_true",
                     help="a mode of its own: Pafutar beside GPT-2 at equal layer sizes (prefill and decode)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default=None, help="with --designs: one size only")
-    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64")
+    ap.add_argument("--design-only", default=None, help="with --designs: one of gpt2, pafutar, pafutar_window_512_keep_64, ruzolorn, ruzolorn_window_512")
     a = ap.parse_args()
     if a.designs:
         if a.gpus != 1:

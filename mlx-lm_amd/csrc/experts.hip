@@ -7,6 +7,14 @@
 //                   wave a feature: act[t, j, :] = w_tj silu(Wg_e x_t) * (Wu_e x_t), then
 //                   y[t, :] += sum_j Wd_e act[t, j, :] + sum_(j: e is an identity expert) w_tj x_t.
 //                   Only the chosen experts' weights are read: the kernels for few tokens.
+//   expert_tiles    the same for many tokens: the picks are sorted by expert on the device
+//                   (expert_sort: counts, offsets, tiles of up to 64 picks of one expert), and
+//                   every tile is a small matrix product on the matrix cores with the rows
+//                   gathered through the sorted list: [gate | up] with the activation and the
+//                   pick's weight in the epilogue, then down into a row of its own for every
+//                   pick; expert_combine adds a token's picks in their order, and the identity
+//                   experts' share.  The grid is as large as the tiles could be at most; blocks
+//                   beyond the tiles that there are leave at once, so nothing comes to the host.
 // The router's softmax, the choice and the weights are 32-bit; products accumulate in 32-bit.
 #include "common.h"
 
@@ -110,6 +118,191 @@ __global__ __launch_bounds__(256) void expert_rows_down_kernel(const T* __restri
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// many tokens: picks sorted by expert, a tile of picks a block
+
+#define TILE_PICKS 64
+
+// One block.  tiles: (expert, first place in `order`, picks) each.
+__global__ __launch_bounds__(1024) void expert_sort_kernel(const int* __restrict__ idx, int n_items, int n_experts,
+                                                           int* __restrict__ order, int* __restrict__ tiles,
+                                                           int* __restrict__ n_tiles) {
+  extern __shared__ int lds_i[];
+  int* counts = lds_i;
+  int* cursor = lds_i + n_experts;
+  for (int e = threadIdx.x; e < n_experts; e += 1024) counts[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_items; i += 1024) {
+    const int e = idx[i];
+    if (e < n_experts) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      cursor[e] = at;
+      for (int r0 = 0; r0 < counts[e]; r0 += TILE_PICKS) {
+        tiles[3 * nt] = e, tiles[3 * nt + 1] = at + r0, tiles[3 * nt + 2] = min(TILE_PICKS, counts[e] - r0);
+        ++nt;
+      }
+      at += counts[e];
+    }
+    *n_tiles = nt;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_items; i += 1024) {
+    const int e = idx[i];
+    if (e < n_experts) order[atomicAdd(&cursor[e], 1)] = i;  // (any order within an expert: a pick's row is computed by itself)
+  }
+}
+
+// A lane's share of a 16 x 16 product's operands: row (or column) lane % 16, KL values of k from
+// KL * (lane / 16) on; the sums land as rows 4 (lane / 16) + i, column lane % 16.
+template <typename T>
+struct Frag;
+template <>
+struct Frag<bf16> {
+  typedef bf16x8_t V;
+  static constexpr int KL = 8;
+  // (a lane beyond K brings zeros: the matrix instruction takes every lane's registers, whatever
+  // the lanes' state, so the product itself must not stand under a condition)
+  static __device__ __forceinline__ V load(const bf16* p, bool inside) {
+    u32x4_t bits = {0u, 0u, 0u, 0u};
+    if (inside) bits = *(const u32x4_t*)p;
+    return __builtin_bit_cast(bf16x8_t, bits);
+  }
+  static __device__ __forceinline__ f32x4_t mma(V a, V b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Frag<float> {
+  typedef f32x4_t V;
+  static constexpr int KL = 4;
+  static __device__ __forceinline__ V load(const float* p, bool inside) {
+    f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+    if (inside) v = *(const f32x4_t*)p;
+    return v;
+  }
+  static __device__ __forceinline__ f32x4_t mma(V a, V b, f32x4_t c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, c, 0, 0, 0);
+  }
+};
+
+// Block (tile, 64 features): a wave 16 picks x 64 features of gate and of up, operands straight
+// from memory.  act[pick, f] = weight * silu(gate) * up.
+template <typename T>
+__global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w_gate,
+                                                              const T* __restrict__ w_up, const int* __restrict__ order,
+                                                              const int* __restrict__ tiles, const int* __restrict__ n_tiles,
+                                                              const float* __restrict__ weight, int top, int F, int width,
+                                                              T* __restrict__ act) {
+  typedef Frag<T> Fr;
+  if ((int)blockIdx.x >= *n_tiles) return;
+  const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
+  if (16 * wave >= count) return;  // (no barrier in this kernel)
+  const int item = order[first + min(16 * wave + r, count - 1)];
+  const T* xrow = x + (size_t)(item / top) * ldx;
+  const int f0 = blockIdx.y * 64;
+  const T* grow[4];
+  const T* urow[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const size_t f = (size_t)e * F + min(f0 + 16 * c + r, F - 1);
+    grow[c] = w_gate + f * width, urow[c] = w_up + f * width;
+  }
+  f32x4_t ag[4], au[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) ag[c] = au[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < width; k0 += 4 * Fr::KL) {
+    const int k = k0 + Fr::KL * g;
+    const bool inside = k < width;  // (the width is a multiple of KL: a lane's values are all inside or all outside)
+    const typename Fr::V a = Fr::load(xrow + k, inside);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      ag[c] = Fr::mma(a, Fr::load(grow[c] + k, inside), ag[c]);
+      au[c] = Fr::mma(a, Fr::load(urow[c] + k, inside), au[c]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ri = 16 * wave + 4 * g + i;
+    if (ri >= count) continue;
+    const int it = order[first + ri];
+    const float wt = weight[it];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int f = f0 + 16 * c + r;
+      if (f < F) act[(size_t)it * F + f] = from_f32<T>(wt * silu_f(ag[c][i]) * au[c][i]);
+    }
+  }
+}
+
+// Block (tile, 64 columns): out[pick, n] = sum_f act[pick, f] w_down[e, n, f].
+template <typename T>
+__global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
+                                                                const int* __restrict__ order, const int* __restrict__ tiles,
+                                                                const int* __restrict__ n_tiles, int F, int width,
+                                                                float* __restrict__ out) {
+  typedef Frag<T> Fr;
+  if ((int)blockIdx.x >= *n_tiles) return;
+  const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
+  if (16 * wave >= count) return;
+  const T* arow = act + (size_t)order[first + min(16 * wave + r, count - 1)] * F;
+  const int n0 = blockIdx.y * 64;
+  const T* drow[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) drow[c] = w_down + ((size_t)e * width + min(n0 + 16 * c + r, width - 1)) * F;
+  f32x4_t acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < F; k0 += 4 * Fr::KL) {
+    const int k = k0 + Fr::KL * g;
+    const bool inside = k < F;
+    const typename Fr::V a = Fr::load(arow + k, inside);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = Fr::mma(a, Fr::load(drow[c] + k, inside), acc[c]);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ri = 16 * wave + 4 * g + i;
+    if (ri >= count) continue;
+    const size_t it = order[first + ri];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int n = n0 + 16 * c + r;
+      if (n < width) out[it * width + n] = acc[c][i];
+    }
+  }
+}
+
+// Thread (token, column): a token's picks in their order, identity experts give weight * x.
+template <typename T>
+__global__ __launch_bounds__(256) void expert_combine_kernel(const float* __restrict__ out, const int* __restrict__ idx,
+                                                             const float* __restrict__ weight, const T* __restrict__ x, int ldx,
+                                                             int n_experts, int top, int width, float* __restrict__ y, int ldy,
+                                                             int accumulate) {
+  const int n = blockIdx.y * 256 + threadIdx.x, t = blockIdx.x;
+  if (n >= width) return;
+  float s = 0.f, same = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const size_t it = (size_t)t * top + j;
+    if (idx[it] >= n_experts)
+      same += weight[it];
+    else
+      s += out[it * width + n];
+  }
+  const float v = s + same * to_f32(x[(size_t)t * ldx + n]);
+  float* o = y + (size_t)t * ldy + n;
+  *o = accumulate ? *o + v : v;
+}
+
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 extern "C" int router_choice(const float* z, int ldz, const float* correction, int n_tokens, int n_out, int top,
@@ -162,5 +355,50 @@ extern "C" int expert_rows(const void* x, int ldx, const void* w_gate, const voi
     RUN(bf16);
 #undef RUN
   CHECK_LAUNCH("expert_rows");
+  return 0;
+}
+
+// The most tiles that n_items picks over n_experts experts can make.
+extern "C" int expert_tiles_most(int n_items, int n_experts) { return (n_items + TILE_PICKS - 1) / TILE_PICKS + n_experts; }
+
+// 1 if expert_tiles takes these sizes (the operands are read 16 bytes a lane).
+extern "C" int expert_tiles_takes(int F, int width, int dtype) {
+  const int kl = dtype == DT_BF16 ? 8 : 4;
+  return F > 0 && F % kl == 0 && width % kl == 0;
+}
+
+// order: [n_tokens * top] ints, tiles: [3 * expert_tiles_most] ints, n_tiles: one int, act: [n_tokens * top, F]
+// of the compute dtype, out: [n_tokens * top, width] floats.
+extern "C" int expert_tiles(const void* x, int ldx, const void* w_gate, const void* w_up, const void* w_down, const int* idx,
+                            const float* weight, int n_tokens, int n_experts, int top, int F, int width, int* order, int* tiles,
+                            int* n_tiles, void* act, float* out, float* y, int ldy, int accumulate, int dtype,
+                            hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (!x || !idx || !weight || !y || !w_gate || !w_up || !w_down || !order || !tiles || !n_tiles || !act || !out)
+    FAIL("expert_tiles: null pointer");
+  if (n_experts <= 0 || top <= 0 || ldx < width || ldy < width) FAIL("expert_tiles: sizes");
+  if (dtype != DT_F32 && dtype != DT_BF16) FAIL("expert_tiles: unknown dtype code %d", dtype);
+  if (!expert_tiles_takes(F, width, dtype)) FAIL("expert_tiles: inner size %d and width %d must be multiples of %d", F, width, dtype == DT_BF16 ? 8 : 4);
+  if (n_experts > 8192) FAIL("expert_tiles: %d experts are more than the sorting block's LDS holds", n_experts);
+  if (ldx % (dtype == DT_BF16 ? 8 : 4) || ((uintptr_t)x & 15)) FAIL("expert_tiles: the rows of x must be 16-byte aligned");
+  const int n_items = n_tokens * top, most = expert_tiles_most(n_items, n_experts);
+  hipLaunchKernelGGL(expert_sort_kernel, dim3(1), dim3(1024), 2 * n_experts * sizeof(int), stream, idx, n_items, n_experts,
+                     order, tiles, n_tiles);
+  dim3 block(256), up_grid(most, (F + 63) / 64), down_grid(most, (width + 63) / 64), sum_grid(n_tokens, (width + 255) / 256);
+#define RUN(T)                                                                                                          \
+  do {                                                                                                                  \
+    hipLaunchKernelGGL(expert_tiles_up_kernel<T>, up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,        \
+                       (const T*)w_up, order, tiles, n_tiles, weight, top, F, width, (T*)act);                          \
+    hipLaunchKernelGGL(expert_tiles_down_kernel<T>, down_grid, block, 0, stream, (const T*)act, (const T*)w_down, order, \
+                       tiles, n_tiles, F, width, out);                                                                  \
+    hipLaunchKernelGGL(expert_combine_kernel<T>, sum_grid, block, 0, stream, out, idx, weight, (const T*)x, ldx,        \
+                       n_experts, top, width, y, ldy, accumulate);                                                      \
+  } while (0)
+  if (dtype == DT_F32)
+    RUN(float);
+  else
+    RUN(bf16);
+#undef RUN
+  CHECK_LAUNCH("expert_tiles");
   return 0;
 }

@@ -123,6 +123,193 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
   for (int i = tid; i < N * P; i += 256) Sg[i] = S[i];
 }
 
+// The same recurrence a chunk of C tokens at a time, for portions of many tokens: with
+// L_t = log a_1 + ... + log a_t inside the chunk,
+//   o_t = exp(L_t) S_0^T q_t + sum_(j <= t) exp(L_t - L_j) (q_t . k_j) v_j
+//   S_C = exp(L_C) S_0 + sum_j exp(L_C - L_j) k_j v_j^T
+// so a chunk is four small matrix products (q k^T, that times v, q S_0, k^T v) whose sums run over
+// tokens side by side instead of one token after the other; every exponent is <= 0.  All in LDS,
+// 32-bit, 4 x 4 outputs a thread: QT, KT [Np][C + 4] (transposed, so that four tokens are one
+// 16-byte read), KW [C][Np] (keys times their decay to the chunk's end), V, O [C][Pp], AT [C][C + 4],
+// S [Np][Pp]; Np, Pp: the head sizes rounded up to four, the padding zero.
+template <typename T>
+__global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
+  extern __shared__ float lds[];
+  __shared__ float Lc[64];
+  const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
+  const int h = blockIdx.x, r = blockIdx.y, hk = h / (a.H / a.Hk);
+  float* QT = lds;
+  float* KT = QT + (size_t)Np * CP;
+  float* KW = KT + (size_t)Np * CP;
+  float* V = KW + (size_t)C * Np;
+  float* O = V + (size_t)C * Pp;
+  float* AT = O + (size_t)C * Pp;
+  float* S = AT + (size_t)C * CP;
+  const int start = a.seq_start[r], n = a.seq_len[r];
+  float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P;
+  for (int i = tid; i < Np * Pp; i += 256) {
+    const int kn = i / Pp, p = i % Pp;
+    S[i] = kn < N && p < P ? Sg[(size_t)kn * P + p] : 0.f;
+  }
+  const int half = a.rot_dims / 2;
+  const float log_decay = a.log_a ? 0.f : logf(a.decay[h]);
+  for (int c0 = 0; c0 < n; c0 += C) {
+    const int m = min(C, n - c0);
+    const size_t row0 = (size_t)(start + c0);
+    __syncthreads();  // the chunk before is done with every array (and S is loaded)
+    if (tid < C) {
+      float acc = 0.f;  // (each of C threads adds its own prefix: C is at most 64)
+      for (int t = 0; t <= tid && t < m; ++t) acc += a.log_a ? a.log_a[(row0 + t) * a.H + h] : log_decay;
+      Lc[tid] = acc;
+    }
+    // queries and keys, turned and scaled, transposed; a pair of turning columns is one item
+    const int items = N - half;  // pairs (i, i + half) for i < half, then the columns from rot_dims on
+    for (int e = tid; e < C * items; e += 256) {
+      const int t = e / items, it = e % items;
+      float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
+      const int i = it < half ? it : it + half;
+      if (t < m) {
+        const float* qr = a.q + (row0 + t) * a.ldq + (size_t)hk * N;
+        const float* kr = a.k + (row0 + t) * a.ldk + (size_t)hk * N;
+        const float ksc = a.k_mult * (a.k_scale ? a.k_scale[(row0 + t) * a.H + h] : 1.0f);
+        if (it < half) {
+          float sn, cs;
+          sincosf((float)a.positions[row0 + t] * a.inv_freq[it], &sn, &cs);
+          const float qa = qr[it], qb = qr[it + half], ka = kr[it], kb = kr[it + half];
+          q0 = qa * cs - qb * sn, q1 = qb * cs + qa * sn;
+          k0 = (ka * cs - kb * sn) * ksc, k1 = (kb * cs + ka * sn) * ksc;
+        } else {
+          q0 = qr[i], k0 = kr[i] * ksc;
+        }
+      }
+      QT[(size_t)i * CP + t] = q0, KT[(size_t)i * CP + t] = k0;
+      if (it < half) QT[(size_t)(it + half) * CP + t] = q1, KT[(size_t)(it + half) * CP + t] = k1;
+    }
+    for (int e = tid; e < C * (Np - N); e += 256) {  // the padding
+      const int t = e / (Np - N), i = N + e % (Np - N);
+      QT[(size_t)i * CP + t] = 0.f, KT[(size_t)i * CP + t] = 0.f;
+    }
+    for (int e = tid; e < C * Pp; e += 256) {
+      const int t = e / Pp, p = e % Pp;
+      V[e] = t < m && p < P ? a.v[(row0 + t) * a.ldv + (size_t)h * P + p] : 0.f;
+    }
+    __syncthreads();
+    const float L_end = Lc[m - 1];
+    for (int e = tid; e < C * Np; e += 256) {
+      const int j = e / Np, i = e % Np;
+      KW[e] = j < m ? KT[(size_t)i * CP + j] * expf(L_end - Lc[j]) : 0.f;
+    }
+    // AT[j][t] = (q_t . k_j) exp(L_t - L_j) for j <= t, else 0
+    const int ct = C / 4;
+    for (int tile = tid; tile < ct * ct; tile += 256) {
+      const int t0 = (tile / ct) * 4, j0 = (tile % ct) * 4;
+      float acc[4][4] = {};
+      if (j0 <= t0 + 3) {
+        for (int i = 0; i < Np; ++i) {
+          const float4 qv = *(const float4*)(QT + (size_t)i * CP + t0);
+          const float4 kv = *(const float4*)(KT + (size_t)i * CP + j0);
+          const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, ks[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+          for (int x = 0; x < 4; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y) acc[x][y] += qs[x] * ks[y];
+        }
+      }
+#pragma unroll
+      for (int y = 0; y < 4; ++y) {
+        float4 o;
+        float* ov = &o.x;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int t = t0 + x, j = j0 + y;
+          ov[x] = j <= t && t < m ? acc[x][y] * expf(Lc[t] - Lc[j]) : 0.f;
+        }
+        *(float4*)(AT + (size_t)(j0 + y) * CP + t0) = o;
+      }
+    }
+    __syncthreads();
+    // O[t][p] = sum_j AT[j][t] V[j][p] + exp(L_t) sum_i QT[i][t] S[i][p]  (+ skip v)
+    const int pt = Pp / 4;
+    for (int tile = tid; tile < ct * pt; tile += 256) {
+      const int t0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
+      float acc[4][4] = {}, old[4][4] = {};
+      const int j_end = min(m, t0 + 4);
+      for (int j = 0; j < j_end; ++j) {
+        const float4 av = *(const float4*)(AT + (size_t)j * CP + t0);
+        const float4 vv = *(const float4*)(V + (size_t)j * Pp + p0);
+        const float as[4] = {av.x, av.y, av.z, av.w}, vs[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+          for (int y = 0; y < 4; ++y) acc[x][y] += as[x] * vs[y];
+      }
+      for (int i = 0; i < Np; ++i) {
+        const float4 qv = *(const float4*)(QT + (size_t)i * CP + t0);
+        const float4 sv = *(const float4*)(S + (size_t)i * Pp + p0);
+        const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, ss[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+          for (int y = 0; y < 4; ++y) old[x][y] += qs[x] * ss[y];
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const float grow = expf(Lc[min(t0 + x, m - 1)]);
+        float4 o;
+        float* ov = &o.x;
+#pragma unroll
+        for (int y = 0; y < 4; ++y) {
+          ov[y] = acc[x][y] + grow * old[x][y];
+          if (a.skip) ov[y] += a.skip[h] * V[(size_t)(t0 + x) * Pp + p0 + y];
+        }
+        *(float4*)(O + (size_t)(t0 + x) * Pp + p0) = o;
+      }
+    }
+    __syncthreads();
+    // S = exp(L_end) S + KW^T V
+    const float shrink = expf(L_end);
+    const int nt = Np / 4;
+    for (int tile = tid; tile < nt * pt; tile += 256) {
+      const int i0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
+      float acc[4][4] = {};
+      for (int j = 0; j < m; ++j) {
+        const float4 kv = *(const float4*)(KW + (size_t)j * Np + i0);
+        const float4 vv = *(const float4*)(V + (size_t)j * Pp + p0);
+        const float ks[4] = {kv.x, kv.y, kv.z, kv.w}, vs[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+#pragma unroll
+          for (int y = 0; y < 4; ++y) acc[x][y] += ks[x] * vs[y];
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        float4* sp = (float4*)(S + (size_t)(i0 + x) * Pp + p0);
+        float4 sv = *sp;
+        sv.x = shrink * sv.x + acc[x][0], sv.y = shrink * sv.y + acc[x][1];
+        sv.z = shrink * sv.z + acc[x][2], sv.w = shrink * sv.w + acc[x][3];
+        *sp = sv;
+      }
+    }
+    // the rows on their way out: a wave a token
+    for (int t = wave; t < m; t += 4) {
+      float rstd = 1.f;
+      if (a.unit_rms) {
+        float ss = 0.f;
+        for (int p = lane; p < P; p += 64) ss += O[(size_t)t * Pp + p] * O[(size_t)t * Pp + p];
+        rstd = 1.0f / sqrtf(wave_sum(ss) / (float)P + a.eps);
+      }
+      for (int p = lane; p < P; p += 64) {
+        float o = O[(size_t)t * Pp + p] * rstd;
+        if (a.gate) o *= silu_f(a.gate[(row0 + t) * a.ldg + (size_t)h * P + p]);
+        ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + p] = from_f32<T>(o);
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < N * P; i += 256) Sg[i] = S[(size_t)(i / P) * Pp + i % P];
+}
+
 // ---------------------------------------------------------------------------
 
 // Thread (token row, channel c): c < C is a convolution channel, C <= c < C + H a head's step size.
@@ -194,7 +381,15 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define SCAN_MAX_LDS (152 * 1024)
 
-extern "C" int state_scan(const ScanArgs* args, hipStream_t stream) {
+// Floats of LDS that the chunked kernel needs for chunks of C tokens.
+static size_t chunk_floats(int N, int P, int C) {
+  const size_t Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
+  return 2 * Np * CP + (size_t)C * Np + 2 * (size_t)C * Pp + (size_t)C * CP + Np * Pp;
+}
+
+// `chunked`: the kernel that takes a chunk of tokens at a time (for steps in which some request
+// brings many tokens); otherwise, or where not even chunks of 16 fit the LDS, token by token.
+extern "C" int state_scan(const ScanArgs* args, int chunked, hipStream_t stream) {
   const ScanArgs& a = *args;
   if (a.n_requests <= 0 || a.H <= 0) return 0;
   if (!a.q || !a.k || !a.v || !a.out || !a.state || !a.seq_start || !a.seq_len || !a.slot_ids)
@@ -217,6 +412,25 @@ extern "C" int state_scan(const ScanArgs* args, hipStream_t stream) {
     raised = true;
   }
   dim3 grid(a.H, a.n_requests), block(256);
+  int C = 0;
+  if (chunked)
+    for (int c = 64; c >= 16 && !C; c /= 2)
+      if (chunk_floats(a.N, a.P, c) * sizeof(float) <= SCAN_MAX_LDS) C = c;
+  if (C) {
+    static bool chunks_raised = false;
+    if (!chunks_raised) {
+      (void)hipFuncSetAttribute((const void*)state_chunks_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+      (void)hipFuncSetAttribute((const void*)state_chunks_kernel<bf16>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
+      chunks_raised = true;
+    }
+    const size_t bytes = chunk_floats(a.N, a.P, C) * sizeof(float);
+    if (a.out_dtype == DT_F32)
+      hipLaunchKernelGGL(state_chunks_kernel<float>, grid, block, bytes, stream, a, C);
+    else
+      hipLaunchKernelGGL(state_chunks_kernel<bf16>, grid, block, bytes, stream, a, C);
+    CHECK_LAUNCH("state_scan");
+    return 0;
+  }
   if (a.out_dtype == DT_F32)
     hipLaunchKernelGGL(state_scan_kernel<float>, grid, block, lds, stream, a);
   else

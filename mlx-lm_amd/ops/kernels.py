@@ -886,14 +886,15 @@ def _f32_rows(t, name, min_cols):
 
 def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, n_requests, n_heads, n_key_heads,
                key_dim, value_dim, log_a=None, decay=None, k_scale=None, k_mult=1.0, skip=None, rot_dims=0,
-               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None):
+               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None, chunked=False):
     """``S = a S + k v^T; o = S^T q`` token by token for every (request, head), from and into the
     requests' rows of ``state`` (float32 ``[slots, floats a request]``, head ``h``'s matrix
     ``[key_dim, value_dim]`` at ``state_offset + h * key_dim * value_dim``).  ``q``, ``k``
     (``[tokens, >= n_key_heads * key_dim]``), ``v`` (``[tokens, >= n_heads * value_dim]``) and
     ``gate`` are float32 rows (column views of a projection's output are fine); ``out`` is
-    ``[tokens, n_heads * value_dim]`` in float32 or bfloat16.  See csrc/linear_state.hip for the
-    options."""
+    ``[tokens, n_heads * value_dim]`` in float32 or bfloat16.  ``chunked``: the kernel that takes
+    up to 64 tokens of a request at a time (for steps in which a request brings many); otherwise
+    token by token.  See csrc/linear_state.hip for the options."""
     lib = build.load("linear_state")
     a = ScanArgs()
     T = out.shape[0]
@@ -932,7 +933,7 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
         _need(t.numel() >= n_requests, f"state_scan: {name} is shorter than the requests")
         setattr(a, name, t.data_ptr())
     a.n_requests, a.H, a.Hk, a.N, a.P = int(n_requests), int(n_heads), int(n_key_heads), int(key_dim), int(value_dim)
-    rc = lib.state_scan(ctypes.byref(a), _stream())
+    rc = lib.state_scan(ctypes.byref(a), _c_int(int(bool(chunked))), _stream())
     build.check(lib, rc, "state_scan")
     return out
 
@@ -1051,4 +1052,37 @@ def expert_rows(y, x, w_gate, w_up, w_down, idx, weight, top, act, accumulate=Tr
                          _c_int(T), _c_int(n_experts), _c_int(top), _c_int(F), _c_int(width), _ptr(act), _ptr(y),
                          _c_int(ldy), _c_int(int(bool(accumulate))), _c_int(DT[x.dtype]), _stream())
     build.check(lib, rc, "expert_rows")
+    return y
+
+
+def expert_tiles_takes(inner, width, dtype):
+    """Whether ``expert_tiles`` takes experts of this inner size at this width."""
+    return bool(build.load("experts").expert_tiles_takes(_c_int(inner), _c_int(width), _c_int(DT[dtype])))
+
+
+def expert_tiles(y, x, w_gate, w_up, w_down, idx, weight, top, alloc, accumulate=True):
+    """What ``expert_rows`` computes, for many tokens: the picks are sorted by expert on the device
+    and every tile of up to 64 picks of one expert is a small product on the matrix cores.
+    ``alloc(shape, dtype)`` gives the work memory (the sorted list, the tiles, the activations
+    and a float32 row for every pick)."""
+    lib = build.load("experts")
+    ldx, ldy = _rows2d(x, "x"), _rows2d(y, "y")
+    T, width = x.shape
+    n_experts, F = w_gate.shape[0], w_gate.shape[1]
+    _need(y.dtype == torch.float32 and tuple(y.shape) == (T, width) and x.dtype in DT, "expert_tiles: x / y")
+    for name, t, shape in (("w_gate", w_gate, (n_experts, F, width)), ("w_up", w_up, (n_experts, F, width)),
+                           ("w_down", w_down, (n_experts, width, F))):
+        _dev(t, name, x.dtype)
+        _need(tuple(t.shape) == shape, f"expert_tiles: {name} is {tuple(t.shape)}, want {shape}")
+    _dev(idx, "idx", torch.int32)
+    _dev(weight, "weight", torch.float32)
+    _need(idx.numel() >= T * top and weight.numel() >= T * top, "expert_tiles: idx / weight too short")
+    most = lib.expert_tiles_most(_c_int(T * top), _c_int(n_experts))
+    order, tiles, n_tiles = alloc((T * top,), torch.int32), alloc((3 * most,), torch.int32), alloc((1,), torch.int32)
+    act, out = alloc((T * top, F), x.dtype), alloc((T * top, width), torch.float32)
+    rc = lib.expert_tiles(_ptr(x), _c_int(ldx), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(idx), _ptr(weight), _c_int(T),
+                          _c_int(n_experts), _c_int(top), _c_int(F), _c_int(width), _ptr(order), _ptr(tiles), _ptr(n_tiles),
+                          _ptr(act), _ptr(out), _ptr(y), _c_int(ldy), _c_int(int(bool(accumulate))), _c_int(DT[x.dtype]),
+                          _stream())
+    build.check(lib, rc, "expert_tiles")
     return y

@@ -19,14 +19,17 @@ class GatedExperts(FeedForward):
     * ``shared_inner > 0``: one more expert of that inner size (``shared.gate`` ...) that every
       token uses with weight one.
 
-    The choice runs on the device (csrc/experts.hip), so a step launches kernels only.  The chosen
-    experts' weights are read straight from the stacked tensors by kernels that touch nothing
-    else; the shared expert goes through the framework's products.  No counterpart in
+    The choice runs on the device (csrc/experts.hip), so a step launches kernels only.  For few
+    tokens the chosen experts' weights are read straight from the stacked tensors, a wave a
+    feature, by kernels that touch nothing else; for many tokens the picks are sorted by expert on
+    the device and go to the matrix cores in tiles of up to 64 picks of one expert.  The shared
+    expert goes through the framework's products.  No counterpart in
     mlx_lm/models/gpt2.py, whose feed-forward (:71-84) is dense.
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     can_overwrite = True
+    TILES_FROM = 24  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
 
     def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, prefix=""):
         super().__init__(prefix)
@@ -96,9 +99,13 @@ class GatedExperts(FeedForward):
             kernels.silu_mul(act, gu)
             kernels.linear(residual, act, self.shared_out, accumulate=accumulate)
             accumulate = True
-        act = ctx.scratch((T * self.top, self.inner), ctx.dtype) if self.n_experts else None
-        kernels.expert_rows(residual, x, self.w_gate, self.w_up, self.w_down, idx, weight, self.top, act,
-                            accumulate=accumulate)
+        if self.n_experts and T >= self.TILES_FROM and kernels.expert_tiles_takes(self.inner, self.width, x.dtype):
+            kernels.expert_tiles(residual, x, self.w_gate, self.w_up, self.w_down, idx, weight, self.top, ctx.scratch,
+                                 accumulate=accumulate)
+        else:
+            act = ctx.scratch((T * self.top, self.inner), ctx.dtype) if self.n_experts else None
+            kernels.expert_rows(residual, x, self.w_gate, self.w_up, self.w_down, idx, weight, self.top, act,
+                                accumulate=accumulate)
         ctx.scratch_release(mark)
 
 

@@ -12,11 +12,15 @@ class _SequenceArrays:
     start in the flat batch and how many they are (its state row is ``ctx.slot_ids``)."""
 
     step_arrays_key = "sequences"
-    step_array_names = ("starts", "lens")
+    step_array_names = ("starts", "lens", "longest")
+    CHUNKS_FROM = 8  # from this many tokens of one request in a step, the kernel that takes chunks
 
     @staticmethod
     def step_arrays(batch):
-        return {"starts": list(batch.q_starts), "lens": list(batch.q_lens)}
+        return {"starts": list(batch.q_starts), "lens": list(batch.q_lens), "longest": max(batch.q_lens, default=0)}
+
+    def _chunked(self, ctx):
+        return ctx.array("sequences.longest") >= self.CHUNKS_FROM
 
 
 def _matrix(w):
@@ -96,7 +100,8 @@ class Retention(_SequenceArrays, Mixer):
                            ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
                            self.n_heads, self.n_heads, self.key_dim, self.value_dim, decay=self.decay,
                            k_mult=self.key_scale, rot_dims=self.rot_dims, inv_freq=self.inv_freq,
-                           positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:])
+                           positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:],
+                           chunked=self._chunked(ctx))
         kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
         ctx.scratch_release(mark)
 
@@ -179,7 +184,7 @@ class StateSpace(_SequenceArrays, Mixer):
         y = ctx.scratch((T, self.inner), torch.float32)
         kernels.state_scan(y, xbc[:, self.inner + GN:], xbc[:, self.inner:self.inner + GN], xbc[:, :self.inner],
                            cache.state, self.conv_floats, starts, lens, ctx.slot_ids, ctx.n_requests, H, self.groups,
-                           self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip)
+                           self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip, chunked=self._chunked(ctx))
         out = ctx.scratch((T, self.inner), ctx.dtype)
         kernels.gated_group_rmsnorm(out, y, u[:, :self.inner], self.norm_w, self.norm_groups, self.eps)
         kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)

@@ -184,19 +184,23 @@ def _scan_plainly(q, k, v, a, S):
     return torch.stack(out), S
 
 
-@pytest.mark.parametrize("N,P,H,Hk", [(8, 8, 4, 4), (24, 16, 2, 1), (5, 24, 3, 1), (64, 64, 2, 2), (40, 48, 1, 1), (128, 128, 1, 1)])
-def test_the_decaying_state_in_portions_of_two_requests(N, P, H, Hk):
+@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("N,P,H,Hk", [(8, 8, 4, 4), (24, 16, 2, 1), (5, 24, 3, 1), (64, 64, 2, 2), (40, 48, 1, 1), (128, 128, 1, 1),
+                                      (6, 10, 2, 2), (200, 100, 1, 1)])
+def test_the_decaying_state_in_portions_of_two_requests(N, P, H, Hk, chunked):
     """Two requests side by side, three steps: the state rows are read at a portion's start and
-    written at its end, each request's own (rows 2 and 0 of four; the others stay as they are)."""
+    written at its end, each request's own (rows 2 and 0 of four; the others stay as they are).
+    Token by token, and with the kernel that takes a chunk of tokens at a time (portions longer
+    than a chunk, of a chunk and a token, and of one token)."""
     from mlx_lm_amd.ops import kernels
 
     g = torch.Generator().manual_seed(N + P)
-    lens = [[5, 2], [1, 9], [2, 1]]
+    lens = [[5, 2], [1, 9], [2, 1]] if not chunked else [[70, 2], [1, 129], [65, 1]]
     n = [sum(x[0] for x in lens), sum(x[1] for x in lens)]
     q = [torch.randn(m, Hk, N, generator=g).double() for m in n]
     k = [torch.randn(m, Hk, N, generator=g).double() * N ** -0.5 for m in n]
     v = [torch.randn(m, H, P, generator=g).double() for m in n]
-    log_a = [-torch.rand(m, H, generator=g).double() for m in n]
+    log_a = [-torch.rand(m, H, generator=g).double() * (0.1 if chunked else 1.0) for m in n]
     ksc = [torch.rand(m, H, generator=g).double() + 0.5 for m in n]
     skip = torch.randn(H, generator=g)
     state = torch.full((4, 7 + H * N * P), 3.0).cuda()
@@ -214,12 +218,12 @@ def test_the_decaying_state_in_portions_of_two_requests(N, P, H, Hk):
         rows = lambda xs: torch.cat([xs[r][at[r] : at[r] + step[r]].flatten(1) for r in range(2)]).float().cuda()  # noqa: E731
         out = torch.empty(sum(step), H * P, device="cuda")
         kernels.state_scan(out, rows(q), rows(k), rows(v), state, 7, _ints([0, step[0]]), _ints(step), _ints([2, 0]), 2, H, Hk, N, P,
-                           log_a=rows(log_a), k_scale=rows(ksc), skip=skip.cuda())
+                           log_a=rows(log_a), k_scale=rows(ksc), skip=skip.cuda(), chunked=chunked)
         got[0].append(out[: step[0]].cpu()), got[1].append(out[step[0] :].cpu())
         at = [at[0] + step[0], at[1] + step[1]]
     for r in range(2):
         w = want[r].flatten(1)
-        assert (torch.cat(got[r]).double() - w).abs().max() <= 2e-5 * w.abs().max()
+        assert (torch.cat(got[r]).double() - w).abs().max() <= 3e-5 * w.abs().max()
     assert (state[[1, 3]] == 3.0).all() and (state[:, :7] == 3.0).all()
 
 
@@ -249,7 +253,7 @@ def test_a_token_far_back_in_the_decaying_state():
     for a, b in ((0, cut), (cut, n - 1), (n - 1, n)):
         kernels.state_scan(out[a:b], q[a:b].cuda(), k[a:b].cuda(), v[a:b].cuda(), state, 0, _ints([0]), _ints([b - a]), _ints([0]),
                            1, 1, 1, N, P, decay=torch.tensor([decay]).cuda(), k_mult=0.25, rot_dims=N, inv_freq=inv_freq.cuda(),
-                           positions=pos[a:b].to(torch.int32).cuda())
+                           positions=pos[a:b].to(torch.int32).cuda(), chunked=b - a > 8)
     assert (out.double().cpu() - want).abs().max() <= 1e-4 * want.abs().max()
     assert (state.double().cpu().view(N, P) - S).abs().max() <= 1e-4 * S.abs().max()
 
@@ -324,7 +328,7 @@ def test_the_routers_choice(n_out, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,width,F", [(1, 64, 24), (9, 72, 10), (40, 256, 64)])
+@pytest.mark.parametrize("T,width,F", [(1, 64, 24), (9, 72, 10), (40, 256, 64), (300, 72, 40), (70, 104, 8)])
 def test_chosen_experts_and_identity_experts(dtype, T, width, F):
     from mlx_lm_amd.ops import kernels
 
@@ -350,6 +354,15 @@ def test_chosen_experts_and_identity_experts(dtype, T, width, F):
     assert (y.double().cpu() - want).abs().max() <= tol * want.abs().max()
     kernels.expert_rows(y, x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), idx.cuda(), wt.cuda(), top, act, accumulate=False)
     assert (y.double().cpu() - (want - y0.double())).abs().max() <= tol * want.abs().max()
+    if kernels.expert_tiles_takes(F, width, dtype):
+        # the same through the sorted tiles (an expert that no token picked, tiles of fewer than 64 picks)
+        def alloc(shape, dt):
+            return torch.empty(shape, dtype=dt, device="cuda")
+
+        for accumulate in (True, False):
+            y = y0.clone().cuda()
+            kernels.expert_tiles(y, x.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), idx.cuda(), wt.cuda(), top, alloc, accumulate=accumulate)
+            assert (y.double().cpu() - (want if accumulate else want - y0.double())).abs().max() <= tol * want.abs().max()
 
 
 # -- the tests' weights show what they are meant to show ---------------------------------
