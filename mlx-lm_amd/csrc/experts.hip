@@ -20,33 +20,54 @@
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-// A thread a token.  The k-th pick is the largest (choice, lowest index first) below the pick
-// before it, so nothing has to be remembered but the last pick.
+// A wave a token, up to ROUTER_PER_LANE outputs a lane.  The k-th pick is the largest choice score
+// not picked yet, the lowest index on a tie.
+#define ROUTER_PER_LANE 8
 __global__ __launch_bounds__(256) void router_choice_kernel(const float* __restrict__ z, int ldz,
                                                             const float* __restrict__ correction, int n_tokens,
                                                             int n_out, int top, int* __restrict__ idx,
                                                             float* __restrict__ weight) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t >= n_tokens) return;
+  const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= n_tokens) return;  // whole waves leave; no barrier follows
   const float* zr = z + (size_t)t * ldz;
-  float m = zr[0];
-  for (int e = 1; e < n_out; ++e) m = fmaxf(m, zr[e]);
+  float v[ROUTER_PER_LANE], c[ROUTER_PER_LANE];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < ROUTER_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < n_out ? zr[e] : -INFINITY;
+    m = fmaxf(m, v[i]);
+  }
+  m = wave_max(m);
   float sum = 0.f;
-  for (int e = 0; e < n_out; ++e) sum += expf(zr[e] - m);
-  const float inv = 1.0f / sum;
-  float last_c = INFINITY;
-  int last_e = -1;
+#pragma unroll
+  for (int i = 0; i < ROUTER_PER_LANE; ++i) {
+    v[i] = lane + 64 * i < n_out ? expf(v[i] - m) : 0.f;
+    sum += v[i];
+  }
+  const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < ROUTER_PER_LANE; ++i) {
+    const int e = lane + 64 * i;
+    v[i] *= inv;
+    c[i] = e < n_out ? (correction ? v[i] + correction[e] : v[i]) : -INFINITY;
+  }
   for (int j = 0; j < top; ++j) {
-    float best_c = -INFINITY, best_s = 0.f;
-    int best_e = -1;
-    for (int e = 0; e < n_out; ++e) {
-      const float s = expf(zr[e] - m) * inv;
-      const float c = correction ? s + correction[e] : s;
-      const bool after = c < last_c || (c == last_c && e > last_e);  // not picked yet
-      if (after && (best_e < 0 || c > best_c)) best_c = c, best_e = e, best_s = s;
-    }
-    idx[(size_t)t * top + j] = best_e, weight[(size_t)t * top + j] = best_s;
-    last_c = best_c, last_e = best_e;
+    float best = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < ROUTER_PER_LANE; ++i) best = fmaxf(best, c[i]);
+    best = wave_max(best);
+    float first = -1e9f;  // minus the lowest index that holds the best score (indices are exact in a float)
+#pragma unroll
+    for (int i = ROUTER_PER_LANE - 1; i >= 0; --i)
+      if (c[i] == best) first = -(float)(lane + 64 * i);
+    const int e = (int)(-wave_max(first));
+#pragma unroll
+    for (int i = 0; i < ROUTER_PER_LANE; ++i)
+      if (lane + 64 * i == e) {
+        idx[(size_t)t * top + j] = e, weight[(size_t)t * top + j] = v[i];
+        c[i] = -INFINITY;  // picked
+      }
   }
 }
 
@@ -59,8 +80,28 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gu,
   out[(size_t)r * ldo + f] = from_f32<T>(silu_f(to_f32(row[f])) * to_f32(row[F + f]));
 }
 
+// sum_k a[k] b[k] over a lane's share of K: 16 bytes a lane and load where K and both rows allow
+// (VEC), a value a lane otherwise.
+template <typename T, bool VEC>
+__device__ __forceinline__ float lane_dot(const T* __restrict__ a, const T* __restrict__ b, int K, int lane) {
+  float s = 0.f;
+  if (VEC) {
+    constexpr int W = 16 / sizeof(T);
+    for (int k = lane * W; k < K; k += 64 * W) {
+      const u32x4_t av = *(const u32x4_t*)(a + k), bv = *(const u32x4_t*)(b + k);
+      const T* ap = (const T*)&av;
+      const T* bp = (const T*)&bv;
+#pragma unroll
+      for (int i = 0; i < W; ++i) s += to_f32(ap[i]) * to_f32(bp[i]);
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) s += to_f32(a[k]) * to_f32(b[k]);
+  }
+  return s;
+}
+
 // Block (token x pick, feature group): a wave a feature at a time, lanes along the width.
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void expert_rows_up_kernel(const T* __restrict__ x, int ldx,
                                                              const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                              const int* __restrict__ idx,
@@ -74,20 +115,14 @@ __global__ __launch_bounds__(256) void expert_rows_up_kernel(const T* __restrict
   const T* xr = x + (size_t)t * ldx;
   const int f_end = min(F, ((int)blockIdx.y + 1) * feats_a_block);
   for (int f = blockIdx.y * feats_a_block + wave; f < f_end; f += 4) {
-    const T* g = w_gate + ((size_t)e * F + f) * width;
-    const T* u = w_up + ((size_t)e * F + f) * width;
-    float sg = 0.f, su = 0.f;
-    for (int k = lane; k < width; k += 64) {
-      const float xv = to_f32(xr[k]);
-      sg += to_f32(g[k]) * xv, su += to_f32(u[k]) * xv;
-    }
-    sg = wave_sum(sg), su = wave_sum(su);
+    const float sg = wave_sum(lane_dot<T, VEC>(w_gate + ((size_t)e * F + f) * width, xr, width, lane));
+    const float su = wave_sum(lane_dot<T, VEC>(w_up + ((size_t)e * F + f) * width, xr, width, lane));
     if (lane == 0) act[(size_t)item * F + f] = from_f32<T>(wt * silu_f(sg) * su);
   }
 }
 
 // Block (token, column group): a wave an output column at a time, lanes along the features.
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void expert_rows_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
                                                                const int* __restrict__ idx,
                                                                const float* __restrict__ weight,
@@ -105,9 +140,7 @@ __global__ __launch_bounds__(256) void expert_rows_down_kernel(const T* __restri
         same += weight[(size_t)t * top + j];
         continue;
       }
-      const T* d = w_down + ((size_t)e * width + n) * F;
-      const T* a = act + ((size_t)t * top + j) * F;
-      for (int f = lane; f < F; f += 64) s += to_f32(d[f]) * to_f32(a[f]);
+      s += lane_dot<T, VEC>(w_down + ((size_t)e * width + n) * F, act + ((size_t)t * top + j) * F, F, lane);
     }
     s = wave_sum(s);
     if (lane == 0) {
@@ -117,7 +150,6 @@ __global__ __launch_bounds__(256) void expert_rows_down_kernel(const T* __restri
     }
   }
 }
-
 
 // ---------------------------------------------------------------------------
 // many tokens: picks sorted by expert, a tile of picks a block
@@ -310,7 +342,8 @@ extern "C" int router_choice(const float* z, int ldz, const float* correction, i
   if (n_tokens <= 0) return 0;
   if (!z || !idx || !weight) FAIL("router_choice: null pointer");
   if (n_out <= 0 || top <= 0 || top > n_out || ldz < n_out) FAIL("router_choice: %d of %d outputs, rows of %d", top, n_out, ldz);
-  hipLaunchKernelGGL(router_choice_kernel, dim3((n_tokens + 255) / 256), dim3(256), 0, stream, z, ldz, correction,
+  if (n_out > 64 * ROUTER_PER_LANE) FAIL("router_choice: %d outputs, at most %d", n_out, 64 * ROUTER_PER_LANE);
+  hipLaunchKernelGGL(router_choice_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, ldz, correction,
                      n_tokens, n_out, top, idx, weight);
   CHECK_LAUNCH("router_choice");
   return 0;
@@ -339,20 +372,23 @@ extern "C" int expert_rows(const void* x, int ldx, const void* w_gate, const voi
     FAIL("expert_rows: null pointer");
   if (top <= 0 || F <= 0 || width <= 0 || ldx < width || ldy < width) FAIL("expert_rows: sizes");
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("expert_rows: unknown dtype code %d", dtype);
-  const int feats = 16, cols = 16;
+  // (few features and columns a block: a step of one token still puts a block on every CU)
+  const int feats = 8, cols = 8, per = dtype == DT_BF16 ? 8 : 4;
+  const bool vec = F % per == 0 && width % per == 0 && ldx % per == 0 && !((uintptr_t)x & 15);
   dim3 block(256), up_grid(n_tokens * top, (F + feats - 1) / feats), down_grid(n_tokens, (width + cols - 1) / cols);
-#define RUN(T)                                                                                                        \
-  do {                                                                                                                \
-    if (n_experts > 0)                                                                                                \
-      hipLaunchKernelGGL(expert_rows_up_kernel<T>, up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,     \
-                         (const T*)w_up, idx, weight, n_experts, top, F, width, (T*)act, feats);                      \
-    hipLaunchKernelGGL(expert_rows_down_kernel<T>, down_grid, block, 0, stream, (const T*)act, (const T*)w_down, idx, \
-                       weight, (const T*)x, ldx, n_experts, top, F, width, y, ldy, cols, accumulate);                 \
+#define RUN(T, VEC)                                                                                                        \
+  do {                                                                                                                     \
+    if (n_experts > 0)                                                                                                     \
+      hipLaunchKernelGGL((expert_rows_up_kernel<T, VEC>), up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,   \
+                         (const T*)w_up, idx, weight, n_experts, top, F, width, (T*)act, feats);                           \
+    hipLaunchKernelGGL((expert_rows_down_kernel<T, VEC>), down_grid, block, 0, stream, (const T*)act, (const T*)w_down,    \
+                       idx, weight, (const T*)x, ldx, n_experts, top, F, width, y, ldy, cols, accumulate);                 \
   } while (0)
-  if (dtype == DT_F32)
-    RUN(float);
-  else
-    RUN(bf16);
+  if (dtype == DT_F32) {
+    if (vec) RUN(float, true); else RUN(float, false);
+  } else {
+    if (vec) RUN(bf16, true); else RUN(bf16, false);
+  }
 #undef RUN
   CHECK_LAUNCH("expert_rows");
   return 0;

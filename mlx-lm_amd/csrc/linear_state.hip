@@ -132,13 +132,29 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
 // 32-bit, 4 x 4 outputs a thread: QT, KT [Np][C + 4] (transposed, so that four tokens are one
 // 16-byte read), KW [C][Np] (keys times their decay to the chunk's end), V, O [C][Pp], AT [C][C + 4],
 // S [Np][Pp]; Np, Pp: the head sizes rounded up to four, the padding zero.
+//
+// Long portions are cut into spans of `span` tokens that run side by side (SpanArgs.mode): first
+// every span's own contribution to the state, from zero, and its decay (SPAN_STATES); then, a
+// thread an element, the state ahead of every span and the request's new state (span_states_kernel);
+// then every span's outputs from the state ahead of it (SPAN_OUTPUTS).  WHOLE: a request's tokens
+// in one block, chunk after chunk.
+enum { WHOLE = 0, SPAN_STATES = 1, SPAN_OUTPUTS = 2 };
+struct SpanArgs {
+  int mode, span;
+  const int* span_req;    // [spans] the request of a span
+  const int* span_start;  // [spans] its first token, counted from the request's first of this step
+  float* span_state;      // [spans, H, N * P]
+  float* span_decay;      // [spans, H]
+};
+
 template <typename T>
-__global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
+__global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, SpanArgs sp) {
   extern __shared__ float lds[];
   __shared__ float Lc[64];
   const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
-  const int h = blockIdx.x, r = blockIdx.y, hk = h / (a.H / a.Hk);
+  const int h = blockIdx.x, hk = h / (a.H / a.Hk);
+  const int r = sp.mode == WHOLE ? blockIdx.y : sp.span_req[blockIdx.y];
   float* QT = lds;
   float* KT = QT + (size_t)Np * CP;
   float* KW = KT + (size_t)Np * CP;
@@ -146,15 +162,20 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
   float* O = V + (size_t)C * Pp;
   float* AT = O + (size_t)C * Pp;
   float* S = AT + (size_t)C * CP;
-  const int start = a.seq_start[r], n = a.seq_len[r];
-  float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P;
+  const int start = a.seq_start[r];
+  const int lo = sp.mode == WHOLE ? 0 : sp.span_start[blockIdx.y];
+  const int n = sp.mode == WHOLE ? a.seq_len[r] : min(a.seq_len[r], lo + sp.span);
+  float* Sg = sp.mode == WHOLE ? a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P
+                               : sp.span_state + ((size_t)blockIdx.y * a.H + h) * N * P;
   for (int i = tid; i < Np * Pp; i += 256) {
     const int kn = i / Pp, p = i % Pp;
-    S[i] = kn < N && p < P ? Sg[(size_t)kn * P + p] : 0.f;
+    S[i] = sp.mode != SPAN_STATES && kn < N && p < P ? Sg[(size_t)kn * P + p] : 0.f;
   }
   const int half = a.rot_dims / 2;
   const float log_decay = a.log_a ? 0.f : logf(a.decay[h]);
-  for (int c0 = 0; c0 < n; c0 += C) {
+  const bool outputs = sp.mode != SPAN_STATES;
+  float span_log = 0.f;
+  for (int c0 = lo; c0 < n; c0 += C) {
     const int m = min(C, n - c0);
     const size_t row0 = (size_t)(start + c0);
     __syncthreads();  // the chunk before is done with every array (and S is loaded)
@@ -200,9 +221,10 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
       const int j = e / Np, i = e % Np;
       KW[e] = j < m ? KT[(size_t)i * CP + j] * expf(L_end - Lc[j]) : 0.f;
     }
+    span_log += L_end;
     // AT[j][t] = (q_t . k_j) exp(L_t - L_j) for j <= t, else 0
     const int ct = C / 4;
-    for (int tile = tid; tile < ct * ct; tile += 256) {
+    for (int tile = tid; outputs && tile < ct * ct; tile += 256) {
       const int t0 = (tile / ct) * 4, j0 = (tile % ct) * 4;
       float acc[4][4] = {};
       if (j0 <= t0 + 3) {
@@ -231,7 +253,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
     __syncthreads();
     // O[t][p] = sum_j AT[j][t] V[j][p] + exp(L_t) sum_i QT[i][t] S[i][p]  (+ skip v)
     const int pt = Pp / 4;
-    for (int tile = tid; tile < ct * pt; tile += 256) {
+    for (int tile = tid; outputs && tile < ct * pt; tile += 256) {
       const int t0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
       float acc[4][4] = {}, old[4][4] = {};
       const int j_end = min(m, t0 + 4);
@@ -270,7 +292,8 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
     // S = exp(L_end) S + KW^T V
     const float shrink = expf(L_end);
     const int nt = Np / 4;
-    for (int tile = tid; tile < nt * pt; tile += 256) {
+    const bool state_needed = sp.mode != SPAN_OUTPUTS || c0 + C < n;  // (a span's outputs: nobody reads the state after its last chunk)
+    for (int tile = tid; state_needed && tile < nt * pt; tile += 256) {
       const int i0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
       float acc[4][4] = {};
       for (int j = 0; j < m; ++j) {
@@ -292,7 +315,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
       }
     }
     // the rows on their way out: a wave a token
-    for (int t = wave; t < m; t += 4) {
+    for (int t = wave; outputs && t < m; t += 4) {
       float rstd = 1.f;
       if (a.unit_rms) {
         float ss = 0.f;
@@ -307,7 +330,27 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C) {
     }
   }
   __syncthreads();
+  if (sp.mode == SPAN_OUTPUTS) return;
   for (int i = tid; i < N * P; i += 256) Sg[i] = S[(size_t)(i / P) * Pp + i % P];
+  if (sp.mode == SPAN_STATES && tid == 0) sp.span_decay[(size_t)blockIdx.y * a.H + h] = expf(span_log);
+}
+
+// Block (head, request), a thread an element of the state: span_state[s] becomes the state ahead
+// of span s, and the request's row its state after the last span.
+__global__ __launch_bounds__(256) void span_states_kernel(ScanArgs a, SpanArgs sp, const int* __restrict__ span_first) {
+  const int h = blockIdx.x, r = blockIdx.y, NP = a.N * a.P;
+  const int first = span_first[r], n_spans = (a.seq_len[r] + sp.span - 1) / sp.span;
+  float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * NP;
+  for (int i = threadIdx.x; i < NP; i += 256) {
+    float s = Sg[i];
+    for (int c = 0; c < n_spans; ++c) {
+      float* own = sp.span_state + ((size_t)(first + c) * a.H + h) * NP + i;
+      const float add = *own;
+      *own = s;
+      s = sp.span_decay[(size_t)(first + c) * a.H + h] * s + add;
+    }
+    Sg[i] = s;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -389,7 +432,13 @@ static size_t chunk_floats(int N, int P, int C) {
 
 // `chunked`: the kernel that takes a chunk of tokens at a time (for steps in which some request
 // brings many tokens); otherwise, or where not even chunks of 16 fit the LDS, token by token.
-extern "C" int state_scan(const ScanArgs* args, int chunked, hipStream_t stream) {
+// `chunked`: 0 token by token; 1 chunks of tokens, a request a block; 2 chunks, the requests cut
+// into spans of `span` tokens that run side by side (n_spans of them: span_req, span_start; the
+// first span of every request in span_first; span_state: room for n_spans * H * N * P floats,
+// span_decay: for n_spans * H).
+extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spans, const int* span_req,
+                          const int* span_start, const int* span_first, float* span_state, float* span_decay,
+                          hipStream_t stream) {
   const ScanArgs& a = *args;
   if (a.n_requests <= 0 || a.H <= 0) return 0;
   if (!a.q || !a.k || !a.v || !a.out || !a.state || !a.seq_start || !a.seq_len || !a.slot_ids)
@@ -424,10 +473,27 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, hipStream_t stream)
       chunks_raised = true;
     }
     const size_t bytes = chunk_floats(a.N, a.P, C) * sizeof(float);
-    if (a.out_dtype == DT_F32)
-      hipLaunchKernelGGL(state_chunks_kernel<float>, grid, block, bytes, stream, a, C);
-    else
-      hipLaunchKernelGGL(state_chunks_kernel<bf16>, grid, block, bytes, stream, a, C);
+    SpanArgs sp = {WHOLE, 0, nullptr, nullptr, nullptr, nullptr};
+#define CHUNKS(GRID)                                                                                \
+  do {                                                                                              \
+    if (a.out_dtype == DT_F32)                                                                      \
+      hipLaunchKernelGGL(state_chunks_kernel<float>, GRID, block, bytes, stream, a, C, sp);         \
+    else                                                                                            \
+      hipLaunchKernelGGL(state_chunks_kernel<bf16>, GRID, block, bytes, stream, a, C, sp);          \
+  } while (0)
+    if (chunked == 2 && n_spans > 0) {
+      if (!span_req || !span_start || !span_first || !span_state || !span_decay) FAIL("state_scan: null pointer among the spans' arrays");
+      if (span < C || span % C) FAIL("state_scan: spans of %d tokens in chunks of %d", span, C);
+      dim3 span_grid(a.H, n_spans);
+      sp = SpanArgs{SPAN_STATES, span, span_req, span_start, span_state, span_decay};
+      CHUNKS(span_grid);
+      hipLaunchKernelGGL(span_states_kernel, grid, block, 0, stream, a, sp, span_first);
+      sp.mode = SPAN_OUTPUTS;
+      CHUNKS(span_grid);
+    } else {
+      CHUNKS(grid);
+    }
+#undef CHUNKS
     CHECK_LAUNCH("state_scan");
     return 0;
   }

@@ -886,7 +886,7 @@ def _f32_rows(t, name, min_cols):
 
 def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, n_requests, n_heads, n_key_heads,
                key_dim, value_dim, log_a=None, decay=None, k_scale=None, k_mult=1.0, skip=None, rot_dims=0,
-               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None, chunked=False):
+               inv_freq=None, positions=None, unit_rms=False, eps=0.0, gate=None, chunked=False, spans=None):
     """``S = a S + k v^T; o = S^T q`` token by token for every (request, head), from and into the
     requests' rows of ``state`` (float32 ``[slots, floats a request]``, head ``h``'s matrix
     ``[key_dim, value_dim]`` at ``state_offset + h * key_dim * value_dim``).  ``q``, ``k``
@@ -894,7 +894,11 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
     ``gate`` are float32 rows (column views of a projection's output are fine); ``out`` is
     ``[tokens, n_heads * value_dim]`` in float32 or bfloat16.  ``chunked``: the kernel that takes
     up to 64 tokens of a request at a time (for steps in which a request brings many); otherwise
-    token by token.  See csrc/linear_state.hip for the options."""
+    token by token.  ``spans``: ``(tokens a span, number of spans, span_req, span_start,
+    span_first, alloc)`` cuts long portions into spans that run side by side (int32 device arrays:
+    the request and the first token of every span, counted from the request's first token of
+    this step, and every request's first span; ``alloc(shape, dtype)`` gives the work memory).
+    See csrc/linear_state.hip for the options."""
     lib = build.load("linear_state")
     a = ScanArgs()
     T = out.shape[0]
@@ -933,7 +937,18 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
         _need(t.numel() >= n_requests, f"state_scan: {name} is shorter than the requests")
         setattr(a, name, t.data_ptr())
     a.n_requests, a.H, a.Hk, a.N, a.P = int(n_requests), int(n_heads), int(n_key_heads), int(key_dim), int(value_dim)
-    rc = lib.state_scan(ctypes.byref(a), _c_int(int(bool(chunked))), _stream())
+    if spans is not None and chunked:
+        span, n_spans, span_req, span_start, span_first, alloc = spans
+        for name, t, n in (("span_req", span_req, n_spans), ("span_start", span_start, n_spans), ("span_first", span_first, n_requests)):
+            _dev(t, name, torch.int32)
+            _need(t.numel() >= n, f"state_scan: {name} too short")
+        ws_state = alloc((n_spans * n_heads * key_dim * value_dim,), torch.float32)
+        ws_decay = alloc((n_spans * n_heads,), torch.float32)
+        rc = lib.state_scan(ctypes.byref(a), _c_int(2), _c_int(span), _c_int(n_spans), _ptr(span_req), _ptr(span_start),
+                            _ptr(span_first), _ptr(ws_state), _ptr(ws_decay), _stream())
+    else:
+        rc = lib.state_scan(ctypes.byref(a), _c_int(int(bool(chunked))), _c_int(0), _c_int(0), None, None, None, None, None,
+                            _stream())
     build.check(lib, rc, "state_scan")
     return out
 

@@ -12,15 +12,30 @@ class _SequenceArrays:
     start in the flat batch and how many they are (its state row is ``ctx.slot_ids``)."""
 
     step_arrays_key = "sequences"
-    step_array_names = ("starts", "lens", "longest")
+    step_array_names = ("starts", "lens", "longest", "span_req", "span_start", "span_first", "n_spans")
     CHUNKS_FROM = 8  # from this many tokens of one request in a step, the kernel that takes chunks
+    SPAN = 64  # tokens of a span; from two spans of one request on, spans run side by side
 
     @staticmethod
     def step_arrays(batch):
-        return {"starts": list(batch.q_starts), "lens": list(batch.q_lens), "longest": max(batch.q_lens, default=0)}
+        span = _SequenceArrays.SPAN
+        span_req, span_start, span_first = [], [], []
+        for r, n in enumerate(batch.q_lens):
+            span_first.append(len(span_req))
+            for lo in range(0, n, span):
+                span_req.append(r)
+                span_start.append(lo)
+        return {"starts": list(batch.q_starts), "lens": list(batch.q_lens), "longest": max(batch.q_lens, default=0),
+                "span_req": span_req, "span_start": span_start, "span_first": span_first, "n_spans": len(span_req)}
 
     def _chunked(self, ctx):
         return ctx.array("sequences.longest") >= self.CHUNKS_FROM
+
+    def _spans(self, ctx):
+        if ctx.array("sequences.longest") < 2 * self.SPAN:
+            return None
+        return (self.SPAN, ctx.array("sequences.n_spans"), ctx.array("sequences.span_req"), ctx.array("sequences.span_start"),
+                ctx.array("sequences.span_first"), ctx.scratch)
 
 
 def _matrix(w):
@@ -101,7 +116,7 @@ class Retention(_SequenceArrays, Mixer):
                            self.n_heads, self.n_heads, self.key_dim, self.value_dim, decay=self.decay,
                            k_mult=self.key_scale, rot_dims=self.rot_dims, inv_freq=self.inv_freq,
                            positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:],
-                           chunked=self._chunked(ctx))
+                           chunked=self._chunked(ctx), spans=self._spans(ctx))
         kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
         ctx.scratch_release(mark)
 
@@ -184,7 +199,8 @@ class StateSpace(_SequenceArrays, Mixer):
         y = ctx.scratch((T, self.inner), torch.float32)
         kernels.state_scan(y, xbc[:, self.inner + GN:], xbc[:, self.inner:self.inner + GN], xbc[:, :self.inner],
                            cache.state, self.conv_floats, starts, lens, ctx.slot_ids, ctx.n_requests, H, self.groups,
-                           self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip, chunked=self._chunked(ctx))
+                           self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip, chunked=self._chunked(ctx),
+                           spans=self._spans(ctx))
         out = ctx.scratch((T, self.inner), ctx.dtype)
         kernels.gated_group_rmsnorm(out, y, u[:, :self.inner], self.norm_w, self.norm_groups, self.eps)
         kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)

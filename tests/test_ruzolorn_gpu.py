@@ -184,7 +184,7 @@ def _scan_plainly(q, k, v, a, S):
     return torch.stack(out), S
 
 
-@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("chunked", [False, True, "spans"])
 @pytest.mark.parametrize("N,P,H,Hk", [(8, 8, 4, 4), (24, 16, 2, 1), (5, 24, 3, 1), (64, 64, 2, 2), (40, 48, 1, 1), (128, 128, 1, 1),
                                       (6, 10, 2, 2), (200, 100, 1, 1)])
 def test_the_decaying_state_in_portions_of_two_requests(N, P, H, Hk, chunked):
@@ -217,8 +217,16 @@ def test_the_decaying_state_in_portions_of_two_requests(N, P, H, Hk, chunked):
     for step in lens:
         rows = lambda xs: torch.cat([xs[r][at[r] : at[r] + step[r]].flatten(1) for r in range(2)]).float().cuda()  # noqa: E731
         out = torch.empty(sum(step), H * P, device="cuda")
+        spans = None
+        if chunked == "spans":  # spans of 64 tokens side by side: (tokens, spans, their requests, their starts, a request's first)
+            req, first, lo = [], [], []
+            for r_, m_ in enumerate(step):
+                first.append(len(req))
+                req += [r_] * ((m_ + 63) // 64)
+                lo += list(range(0, m_, 64))
+            spans = (64, len(req), _ints(req), _ints(lo), _ints(first), lambda shape, dt: torch.empty(shape, dtype=dt, device="cuda"))
         kernels.state_scan(out, rows(q), rows(k), rows(v), state, 7, _ints([0, step[0]]), _ints(step), _ints([2, 0]), 2, H, Hk, N, P,
-                           log_a=rows(log_a), k_scale=rows(ksc), skip=skip.cuda(), chunked=chunked)
+                           log_a=rows(log_a), k_scale=rows(ksc), skip=skip.cuda(), chunked=bool(chunked), spans=spans)
         got[0].append(out[: step[0]].cpu()), got[1].append(out[step[0] :].cpu())
         at = [at[0] + step[0], at[1] + step[1]]
     for r in range(2):
