@@ -225,8 +225,9 @@ struct Frag<float> {
   }
 };
 
-// Block (tile, 64 features): a wave 16 picks x 64 features of gate and of up, operands straight
-// from memory.  act[pick, f] = weight * silu(gate) * up.
+// Block (tile, 256 features): a wave all of the tile's picks (four groups of 16) x 64 features of
+// gate and of up, operands straight from memory; a weight fragment meets up to four fragments of
+// rows.  act[pick, f] = weight * silu(gate) * up.
 template <typename T>
 __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w_gate,
                                                               const T* __restrict__ w_up, const int* __restrict__ order,
@@ -237,10 +238,12 @@ __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restric
   if ((int)blockIdx.x >= *n_tiles) return;
   const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
-  if (16 * wave >= count) return;  // (no barrier in this kernel)
-  const int item = order[first + min(16 * wave + r, count - 1)];
-  const T* xrow = x + (size_t)(item / top) * ldx;
-  const int f0 = blockIdx.y * 64;
+  const int f0 = blockIdx.y * 256 + wave * 64;
+  if (f0 >= F) return;  // (no barrier in this kernel)
+  const int groups = (count + 15) / 16;
+  const T* xrow[4];
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) xrow[rg] = x + (size_t)(order[first + min(16 * rg + r, count - 1)] / top) * ldx;
   const T* grow[4];
   const T* urow[4];
 #pragma unroll
@@ -248,34 +251,47 @@ __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restric
     const size_t f = (size_t)e * F + min(f0 + 16 * c + r, F - 1);
     grow[c] = w_gate + f * width, urow[c] = w_up + f * width;
   }
-  f32x4_t ag[4], au[4];
+  f32x4_t ag[4][4], au[4][4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) ag[c] = au[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ag[rg][c] = au[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < width; k0 += 4 * Fr::KL) {
     const int k = k0 + Fr::KL * g;
     const bool inside = k < width;  // (the width is a multiple of KL: a lane's values are all inside or all outside)
-    const typename Fr::V a = Fr::load(xrow + k, inside);
+    typename Fr::V a[4], bg[4], bu[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      ag[c] = Fr::mma(a, Fr::load(grow[c] + k, inside), ag[c]);
-      au[c] = Fr::mma(a, Fr::load(urow[c] + k, inside), au[c]);
+    for (int rg = 0; rg < 4; ++rg) a[rg] = Fr::load(xrow[rg] + k, inside);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) bg[c] = Fr::load(grow[c] + k, inside), bu[c] = Fr::load(urow[c] + k, inside);
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      if (rg < groups) {  // (the same for every lane of the block)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          ag[rg][c] = Fr::mma(a[rg], bg[c], ag[rg][c]);
+          au[rg][c] = Fr::mma(a[rg], bu[c], au[rg][c]);
+        }
+      }
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int ri = 16 * wave + 4 * g + i;
-    if (ri >= count) continue;
-    const int it = order[first + ri];
-    const float wt = weight[it];
+  for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int f = f0 + 16 * c + r;
-      if (f < F) act[(size_t)it * F + f] = from_f32<T>(wt * silu_f(ag[c][i]) * au[c][i]);
+    for (int i = 0; i < 4; ++i) {
+      const int ri = 16 * rg + 4 * g + i;
+      if (ri >= count) continue;
+      const int it = order[first + ri];
+      const float wt = weight[it];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int f = f0 + 16 * c + r;
+        if (f < F) act[(size_t)it * F + f] = from_f32<T>(wt * silu_f(ag[rg][c][i]) * au[rg][c][i]);
+      }
     }
-  }
 }
 
-// Block (tile, 64 columns): out[pick, n] = sum_f act[pick, f] w_down[e, n, f].
+// Block (tile, 256 columns): out[pick, n] = sum_f act[pick, f] w_down[e, n, f], laid out as above.
 template <typename T>
 __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
                                                                 const int* __restrict__ order, const int* __restrict__ tiles,
@@ -285,33 +301,49 @@ __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restr
   if ((int)blockIdx.x >= *n_tiles) return;
   const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
-  if (16 * wave >= count) return;
-  const T* arow = act + (size_t)order[first + min(16 * wave + r, count - 1)] * F;
-  const int n0 = blockIdx.y * 64;
+  const int n0 = blockIdx.y * 256 + wave * 64;
+  if (n0 >= width) return;
+  const int groups = (count + 15) / 16;
+  const T* arow[4];
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg) arow[rg] = act + (size_t)order[first + min(16 * rg + r, count - 1)] * F;
   const T* drow[4];
 #pragma unroll
   for (int c = 0; c < 4; ++c) drow[c] = w_down + ((size_t)e * width + min(n0 + 16 * c + r, width - 1)) * F;
-  f32x4_t acc[4];
+  f32x4_t acc[4][4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < F; k0 += 4 * Fr::KL) {
     const int k = k0 + Fr::KL * g;
     const bool inside = k < F;
-    const typename Fr::V a = Fr::load(arow + k, inside);
+    typename Fr::V a[4], b[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = Fr::mma(a, Fr::load(drow[c] + k, inside), acc[c]);
-  }
+    for (int rg = 0; rg < 4; ++rg) a[rg] = Fr::load(arow[rg] + k, inside);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int ri = 16 * wave + 4 * g + i;
-    if (ri >= count) continue;
-    const size_t it = order[first + ri];
+    for (int c = 0; c < 4; ++c) b[c] = Fr::load(drow[c] + k, inside);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int n = n0 + 16 * c + r;
-      if (n < width) out[it * width + n] = acc[c][i];
+    for (int rg = 0; rg < 4; ++rg) {
+      if (rg < groups) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[rg][c] = Fr::mma(a[rg], b[c], acc[rg][c]);
+      }
     }
   }
+#pragma unroll
+  for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ri = 16 * rg + 4 * g + i;
+      if (ri >= count) continue;
+      const size_t it = order[first + ri];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int n = n0 + 16 * c + r;
+        if (n < width) out[it * width + n] = acc[rg][c][i];
+      }
+    }
 }
 
 // Thread (token, column): a token's picks in their order, identity experts give weight * x.
@@ -420,7 +452,7 @@ extern "C" int expert_tiles(const void* x, int ldx, const void* w_gate, const vo
   const int n_items = n_tokens * top, most = expert_tiles_most(n_items, n_experts);
   hipLaunchKernelGGL(expert_sort_kernel, dim3(1), dim3(1024), 2 * n_experts * sizeof(int), stream, idx, n_items, n_experts,
                      order, tiles, n_tiles);
-  dim3 block(256), up_grid(most, (F + 63) / 64), down_grid(most, (width + 63) / 64), sum_grid(n_tokens, (width + 255) / 256);
+  dim3 block(256), up_grid(most, (F + 255) / 256), down_grid(most, (width + 255) / 256), sum_grid(n_tokens, (width + 255) / 256);
 #define RUN(T)                                                                                                          \
   do {                                                                                                                  \
     hipLaunchKernelGGL(expert_tiles_up_kernel<T>, up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,        \

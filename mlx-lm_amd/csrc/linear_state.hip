@@ -7,7 +7,8 @@
 //                   steps.  a_t = exp(log_a[t, h]) or the constant decay[h]; k_t is multiplied by
 //                   k_mult and by k_scale[t, h] where given; q and k may turn with the position
 //                   (the first rot_dims columns of a head, column i with column i + rot_dims / 2,
-//                   by position * inv_freq[i]); the key heads may be fewer than the value heads
+//                   by position * inv_freq[i]; the kernels that take chunks turn q and k in place
+//                   first, so the caller must not need them afterwards); the key heads may be fewer than the value heads
 //                   (head h reads key head h / (H / Hk)).  The output may be divided by its root
 //                   mean square over the head and multiplied by silu(gate) on the way out.
 //   ssm_prepare     causal convolution per channel over a request's tokens with the last
@@ -49,6 +50,7 @@ struct ScanArgs {
   const int* seq_len;
   const int* slot_ids;
   int n_requests, H, Hk, N, P;
+  int n_tokens_hint;  // the token rows of q and k (the kernels that take chunks turn them all at once, in place)
 };
 
 // One block a (head, request); the state in LDS as S[i * P + p], thread (part, p) walks its share
@@ -150,7 +152,7 @@ struct SpanArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, SpanArgs sp) {
   extern __shared__ float lds[];
-  __shared__ float Lc[64];
+  __shared__ float Lc[64], Lraw[64];
   const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
   const int h = blockIdx.x, hk = h / (a.H / a.Hk);
@@ -179,11 +181,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
     const int m = min(C, n - c0);
     const size_t row0 = (size_t)(start + c0);
     __syncthreads();  // the chunk before is done with every array (and S is loaded)
-    if (tid < C) {
-      float acc = 0.f;  // (each of C threads adds its own prefix: C is at most 64)
-      for (int t = 0; t <= tid && t < m; ++t) acc += a.log_a ? a.log_a[(row0 + t) * a.H + h] : log_decay;
-      Lc[tid] = acc;
-    }
+    if (tid < C) Lraw[tid] = tid < m ? (a.log_a ? a.log_a[(row0 + tid) * a.H + h] : log_decay) : 0.f;
     // queries and keys, turned and scaled, transposed; a pair of turning columns is one item
     const int items = N - half;  // pairs (i, i + half) for i < half, then the columns from rot_dims on
     for (int e = tid; e < C * items; e += 256) {
@@ -214,6 +212,12 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
     for (int e = tid; e < C * Pp; e += 256) {
       const int t = e / Pp, p = e % Pp;
       V[e] = t < m && p < P ? a.v[(row0 + t) * a.ldv + (size_t)h * P + p] : 0.f;
+    }
+    __syncthreads();
+    if (tid < C) {
+      float acc = 0.f;  // (each of C threads adds its own prefix: C is at most 64)
+      for (int t = 0; t <= tid; ++t) acc += Lraw[t];
+      Lc[tid] = acc;
     }
     __syncthreads();
     const float L_end = Lc[m - 1];
@@ -353,6 +357,25 @@ __global__ __launch_bounds__(256) void span_states_kernel(ScanArgs a, SpanArgs s
   }
 }
 
+// Queries and keys turned in place ahead of the kernels that take chunks (which would otherwise
+// each turn them again): thread (token, key head, pair of columns).
+__global__ __launch_bounds__(256) void rotate_pairs_kernel(float* __restrict__ q, int ldq, float* __restrict__ k, int ldk,
+                                                           const int* __restrict__ positions,
+                                                           const float* __restrict__ inv_freq, int n_tokens, int heads,
+                                                           int N, int half) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)n_tokens * heads * half) return;
+  const int j = e % half, hd = (e / half) % heads;
+  const long t = e / ((long)half * heads);
+  float sn, cs;
+  sincosf((float)positions[t] * inv_freq[j], &sn, &cs);
+  float* qr = q + t * ldq + (size_t)hd * N;
+  float* kr = k + t * ldk + (size_t)hd * N;
+  const float qa = qr[j], qb = qr[j + half], ka = kr[j], kb = kr[j + half];
+  qr[j] = qa * cs - qb * sn, qr[j + half] = qb * cs + qa * sn;
+  kr[j] = ka * cs - kb * sn, kr[j + half] = kb * cs + ka * sn;
+}
+
 // ---------------------------------------------------------------------------
 
 // Thread (token row, channel c): c < C is a convolution channel, C <= c < C + H a head's step size.
@@ -466,6 +489,15 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
     for (int c = 64; c >= 16 && !C; c /= 2)
       if (chunk_floats(a.N, a.P, c) * sizeof(float) <= SCAN_MAX_LDS) C = c;
   if (C) {
+    ScanArgs turned = a;
+    if (a.rot_dims) {
+      // (q and k are the caller's work memory: the projection's rows, which nothing reads after this)
+      const long items = (long)a.n_tokens_hint * a.Hk * (a.rot_dims / 2);
+      if (a.n_tokens_hint <= 0) FAIL("state_scan: the chunked kernels need the number of token rows");
+      hipLaunchKernelGGL(rotate_pairs_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream, (float*)a.q, a.ldq,
+                         (float*)a.k, a.ldk, a.positions, a.inv_freq, a.n_tokens_hint, a.Hk, a.N, a.rot_dims / 2);
+      turned.rot_dims = 0;
+    }
     static bool chunks_raised = false;
     if (!chunks_raised) {
       (void)hipFuncSetAttribute((const void*)state_chunks_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, SCAN_MAX_LDS);
@@ -477,9 +509,9 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
 #define CHUNKS(GRID)                                                                                \
   do {                                                                                              \
     if (a.out_dtype == DT_F32)                                                                      \
-      hipLaunchKernelGGL(state_chunks_kernel<float>, GRID, block, bytes, stream, a, C, sp);         \
+      hipLaunchKernelGGL(state_chunks_kernel<float>, GRID, block, bytes, stream, turned, C, sp);         \
     else                                                                                            \
-      hipLaunchKernelGGL(state_chunks_kernel<bf16>, GRID, block, bytes, stream, a, C, sp);          \
+      hipLaunchKernelGGL(state_chunks_kernel<bf16>, GRID, block, bytes, stream, turned, C, sp);          \
   } while (0)
     if (chunked == 2 && n_spans > 0) {
       if (!span_req || !span_start || !span_first || !span_state || !span_decay) FAIL("state_scan: null pointer among the spans' arrays");
@@ -487,7 +519,7 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
       dim3 span_grid(a.H, n_spans);
       sp = SpanArgs{SPAN_STATES, span, span_req, span_start, span_state, span_decay};
       CHUNKS(span_grid);
-      hipLaunchKernelGGL(span_states_kernel, grid, block, 0, stream, a, sp, span_first);
+      hipLaunchKernelGGL(span_states_kernel, grid, block, 0, stream, turned, sp, span_first);
       sp.mode = SPAN_OUTPUTS;
       CHUNKS(span_grid);
     } else {

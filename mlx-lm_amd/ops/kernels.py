@@ -874,7 +874,7 @@ class ScanArgs(ctypes.Structure):
                 ("gate", _vp), ("ldg", _c_int), ("out", _vp), ("ldo", _c_int), ("out_dtype", _c_int),
                 ("state", _vp), ("state_stride", _c_size_t), ("state_offset", _c_size_t), ("seq_start", _vp),
                 ("seq_len", _vp), ("slot_ids", _vp), ("n_requests", _c_int), ("H", _c_int), ("Hk", _c_int),
-                ("N", _c_int), ("P", _c_int)]
+                ("N", _c_int), ("P", _c_int), ("n_tokens_hint", _c_int)]
 
 
 def _f32_rows(t, name, min_cols):
@@ -891,7 +891,8 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
     requests' rows of ``state`` (float32 ``[slots, floats a request]``, head ``h``'s matrix
     ``[key_dim, value_dim]`` at ``state_offset + h * key_dim * value_dim``).  ``q``, ``k``
     (``[tokens, >= n_key_heads * key_dim]``), ``v`` (``[tokens, >= n_heads * value_dim]``) and
-    ``gate`` are float32 rows (column views of a projection's output are fine); ``out`` is
+    ``gate`` are float32 rows (column views of a projection's output are fine; with ``chunked`` and
+    ``rot_dims`` the rows of ``q`` and ``k`` are turned in place, so they are work memory); ``out`` is
     ``[tokens, n_heads * value_dim]`` in float32 or bfloat16.  ``chunked``: the kernel that takes
     up to 64 tokens of a request at a time (for steps in which a request brings many); otherwise
     token by token.  ``spans``: ``(tokens a span, number of spans, span_req, span_start,
@@ -937,6 +938,7 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
         _need(t.numel() >= n_requests, f"state_scan: {name} is shorter than the requests")
         setattr(a, name, t.data_ptr())
     a.n_requests, a.H, a.Hk, a.N, a.P = int(n_requests), int(n_heads), int(n_key_heads), int(key_dim), int(value_dim)
+    a.n_tokens_hint = int(T)
     if spans is not None and chunked:
         span, n_spans, span_req, span_start, span_first, alloc = spans
         for name, t, n in (("span_req", span_req, n_spans), ("span_start", span_start, n_spans), ("span_first", span_first, n_requests)):

@@ -29,7 +29,7 @@ class GatedExperts(FeedForward):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     can_overwrite = True
-    TILES_FROM = 24  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
+    TILES_FROM = 128  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
 
     def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, prefix=""):
         super().__init__(prefix)
