@@ -256,25 +256,37 @@ __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restric
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
     for (int c = 0; c < 4; ++c) ag[rg][c] = au[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < width; k0 += 4 * Fr::KL) {
-    const int k = k0 + Fr::KL * g;
-    const bool inside = k < width;  // (the width is a multiple of KL: a lane's values are all inside or all outside)
-    typename Fr::V a[4], bg[4], bu[4];
-#pragma unroll
-    for (int rg = 0; rg < 4; ++rg) a[rg] = Fr::load(xrow[rg] + k, inside);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) bg[c] = Fr::load(grow[c] + k, inside), bu[c] = Fr::load(urow[c] + k, inside);
-#pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
-      if (rg < groups) {  // (the same for every lane of the block)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          ag[rg][c] = Fr::mma(a[rg], bg[c], ag[rg][c]);
-          au[rg][c] = Fr::mma(a[rg], bu[c], au[rg][c]);
-        }
-      }
-    }
+  // two sets of operands by turns: the next step's loads are on their way during this step's products
+  // (the width is a multiple of KL: a lane's values are all inside or all outside)
+  typename Fr::V a[2][4], bg[2][4], bu[2][4];
+  const int step = 4 * Fr::KL;
+#define LOAD_SET(S, K0)                                                                                 \
+  do {                                                                                                  \
+    const int k_ = (K0) + Fr::KL * g;                                                                   \
+    const bool in_ = k_ < width;                                                                        \
+    _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) a[S][rg] = Fr::load(xrow[rg] + k_, in_);           \
+    _Pragma("unroll") for (int c = 0; c < 4; ++c) bg[S][c] = Fr::load(grow[c] + k_, in_), bu[S][c] = Fr::load(urow[c] + k_, in_); \
+  } while (0)
+#define MMA_SET(S)                                                                                      \
+  do {                                                                                                  \
+    _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) {                                                  \
+      if (rg < groups) { /* (the same for every lane of the block) */                                   \
+        _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                 \
+          ag[rg][c] = Fr::mma(a[S][rg], bg[S][c], ag[rg][c]);                                           \
+          au[rg][c] = Fr::mma(a[S][rg], bu[S][c], au[rg][c]);                                           \
+        }                                                                                               \
+      }                                                                                                 \
+    }                                                                                                   \
+  } while (0)
+  LOAD_SET(0, 0);
+  for (int k0 = 0; k0 < width; k0 += 2 * step) {
+    LOAD_SET(1, k0 + step);  // (beyond the width: zeros, and nothing is read)
+    MMA_SET(0);
+    LOAD_SET(0, k0 + 2 * step);
+    MMA_SET(1);
   }
+#undef LOAD_SET
+#undef MMA_SET
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
@@ -315,22 +327,32 @@ __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restr
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < F; k0 += 4 * Fr::KL) {
-    const int k = k0 + Fr::KL * g;
-    const bool inside = k < F;
-    typename Fr::V a[4], b[4];
-#pragma unroll
-    for (int rg = 0; rg < 4; ++rg) a[rg] = Fr::load(arow[rg] + k, inside);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) b[c] = Fr::load(drow[c] + k, inside);
-#pragma unroll
-    for (int rg = 0; rg < 4; ++rg) {
-      if (rg < groups) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[rg][c] = Fr::mma(a[rg], b[c], acc[rg][c]);
-      }
-    }
+  typename Fr::V a[2][4], b[2][4];
+  const int step = 4 * Fr::KL;
+#define LOAD_SET(S, K0)                                                                        \
+  do {                                                                                         \
+    const int k_ = (K0) + Fr::KL * g;                                                          \
+    const bool in_ = k_ < F;                                                                   \
+    _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) a[S][rg] = Fr::load(arow[rg] + k_, in_);  \
+    _Pragma("unroll") for (int c = 0; c < 4; ++c) b[S][c] = Fr::load(drow[c] + k_, in_);       \
+  } while (0)
+#define MMA_SET(S)                                                                             \
+  do {                                                                                         \
+    _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) {                                         \
+      if (rg < groups) {                                                                       \
+        _Pragma("unroll") for (int c = 0; c < 4; ++c) acc[rg][c] = Fr::mma(a[S][rg], b[S][c], acc[rg][c]); \
+      }                                                                                        \
+    }                                                                                          \
+  } while (0)
+  LOAD_SET(0, 0);
+  for (int k0 = 0; k0 < F; k0 += 2 * step) {
+    LOAD_SET(1, k0 + step);
+    MMA_SET(0);
+    LOAD_SET(0, k0 + 2 * step);
+    MMA_SET(1);
   }
+#undef LOAD_SET
+#undef MMA_SET
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll

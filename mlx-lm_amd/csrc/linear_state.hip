@@ -131,9 +131,10 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
 //   S_C = exp(L_C) S_0 + sum_j exp(L_C - L_j) k_j v_j^T
 // so a chunk is four small matrix products (q k^T, that times v, q S_0, k^T v) whose sums run over
 // tokens side by side instead of one token after the other; every exponent is <= 0.  All in LDS,
-// 32-bit, 4 x 4 outputs a thread: QT, KT [Np][C + 4] (transposed, so that four tokens are one
-// 16-byte read), KW [C][Np] (keys times their decay to the chunk's end), V, O [C][Pp], AT [C][C + 4],
-// S [Np][Pp]; Np, Pp: the head sizes rounded up to four, the padding zero.
+// 32-bit, on the matrix cores (v_mfma_f32_16x16x4_f32, a wave a tile of 16 x 16): QT, KT
+// [Np][C + 4] (transposed: a wave's operand is sixteen consecutive tokens), KW [C][Np] (keys times
+// their decay to the chunk's end), V, O [C][Pp], AT [C][C + 4], S [Np][Pp]; Np, Pp: the head sizes
+// rounded up to sixteen, the padding zero.
 //
 // Long portions are cut into spans of `span` tokens that run side by side (SpanArgs.mode): first
 // every span's own contribution to the state, from zero, and its decay (SPAN_STATES); then, a
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
   extern __shared__ float lds[];
   __shared__ float Lc[64], Lraw[64];
   const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
+  const int Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
   const int h = blockIdx.x, hk = h / (a.H / a.Hk);
   const int r = sp.mode == WHOLE ? blockIdx.y : sp.span_req[blockIdx.y];
   float* QT = lds;
@@ -226,96 +227,61 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
       KW[e] = j < m ? KT[(size_t)i * CP + j] * expf(L_end - Lc[j]) : 0.f;
     }
     span_log += L_end;
-    // AT[j][t] = (q_t . k_j) exp(L_t - L_j) for j <= t, else 0
-    const int ct = C / 4;
-    for (int tile = tid; outputs && tile < ct * ct; tile += 256) {
-      const int t0 = (tile / ct) * 4, j0 = (tile % ct) * 4;
-      float acc[4][4] = {};
-      if (j0 <= t0 + 3) {
-        for (int i = 0; i < Np; ++i) {
-          const float4 qv = *(const float4*)(QT + (size_t)i * CP + t0);
-          const float4 kv = *(const float4*)(KT + (size_t)i * CP + j0);
-          const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, ks[4] = {kv.x, kv.y, kv.z, kv.w};
+    // The three products run on the matrix cores in 32-bit (v_mfma_f32_16x16x4_f32: lane l brings
+    // A[l % 16][l / 16] and B[l / 16][l % 16] and gets D[4 (l / 16) + x][l % 16]); a wave a tile
+    // of 16 x 16.  AT[j][t] = (q_t . k_j) exp(L_t - L_j) for j <= t, else 0
+    const int ct = C / 16, lr = lane & 15, lg = lane >> 4;
+    for (int tile = wave; outputs && tile < ct * ct; tile += 4) {
+      const int t0 = (tile / ct) * 16, j0 = (tile % ct) * 16;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      if (j0 <= t0 + 15)
+        for (int i = 0; i < Np; i += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(QT[(size_t)(i + lg) * CP + t0 + lr], KT[(size_t)(i + lg) * CP + j0 + lr], acc, 0, 0, 0);
+      // D[m = t][n = j]: this lane holds t = t0 + 4 lg + x for j = j0 + lr
+      const int j = j0 + lr;
+      float4 o;
+      float* ov = &o.x;
 #pragma unroll
-          for (int x = 0; x < 4; ++x)
-#pragma unroll
-            for (int y = 0; y < 4; ++y) acc[x][y] += qs[x] * ks[y];
-        }
+      for (int x = 0; x < 4; ++x) {
+        const int t = t0 + 4 * lg + x;
+        ov[x] = j <= t && t < m ? acc[x] * expf(Lc[t] - Lc[j]) : 0.f;
       }
-#pragma unroll
-      for (int y = 0; y < 4; ++y) {
-        float4 o;
-        float* ov = &o.x;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          const int t = t0 + x, j = j0 + y;
-          ov[x] = j <= t && t < m ? acc[x][y] * expf(Lc[t] - Lc[j]) : 0.f;
-        }
-        *(float4*)(AT + (size_t)(j0 + y) * CP + t0) = o;
-      }
+      *(float4*)(AT + (size_t)j * CP + t0 + 4 * lg) = o;
     }
     __syncthreads();
     // O[t][p] = sum_j AT[j][t] V[j][p] + exp(L_t) sum_i QT[i][t] S[i][p]  (+ skip v)
-    const int pt = Pp / 4;
-    for (int tile = tid; outputs && tile < ct * pt; tile += 256) {
-      const int t0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
-      float acc[4][4] = {}, old[4][4] = {};
-      const int j_end = min(m, t0 + 4);
-      for (int j = 0; j < j_end; ++j) {
-        const float4 av = *(const float4*)(AT + (size_t)j * CP + t0);
-        const float4 vv = *(const float4*)(V + (size_t)j * Pp + p0);
-        const float as[4] = {av.x, av.y, av.z, av.w}, vs[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-#pragma unroll
-          for (int y = 0; y < 4; ++y) acc[x][y] += as[x] * vs[y];
-      }
-      for (int i = 0; i < Np; ++i) {
-        const float4 qv = *(const float4*)(QT + (size_t)i * CP + t0);
-        const float4 sv = *(const float4*)(S + (size_t)i * Pp + p0);
-        const float qs[4] = {qv.x, qv.y, qv.z, qv.w}, ss[4] = {sv.x, sv.y, sv.z, sv.w};
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-#pragma unroll
-          for (int y = 0; y < 4; ++y) old[x][y] += qs[x] * ss[y];
-      }
+    const int pt = Pp / 16;
+    for (int tile = wave; outputs && tile < ct * pt; tile += 4) {
+      const int t0 = (tile / pt) * 16, p0 = (tile % pt) * 16;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, old = {0.f, 0.f, 0.f, 0.f};
+      const int j_end = min((m + 3) & ~3, t0 + 16);  // (AT is zero where j > t or t >= m, V where j >= m)
+      for (int j = 0; j < j_end; j += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(AT[(size_t)(j + lg) * CP + t0 + lr], V[(size_t)(j + lg) * Pp + p0 + lr], acc, 0, 0, 0);
+      for (int i = 0; i < Np; i += 4)
+        old = __builtin_amdgcn_mfma_f32_16x16x4f32(QT[(size_t)(i + lg) * CP + t0 + lr], S[(size_t)(i + lg) * Pp + p0 + lr], old, 0, 0, 0);
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        const float grow = expf(Lc[min(t0 + x, m - 1)]);
-        float4 o;
-        float* ov = &o.x;
-#pragma unroll
-        for (int y = 0; y < 4; ++y) {
-          ov[y] = acc[x][y] + grow * old[x][y];
-          if (a.skip) ov[y] += a.skip[h] * V[(size_t)(t0 + x) * Pp + p0 + y];
-        }
-        *(float4*)(O + (size_t)(t0 + x) * Pp + p0) = o;
+        const int t = t0 + 4 * lg + x, pcol = p0 + lr;
+        float o = acc[x] + expf(Lc[min(t, m - 1)]) * old[x];
+        if (a.skip) o += a.skip[h] * V[(size_t)t * Pp + pcol];
+        O[(size_t)t * Pp + pcol] = o;
       }
     }
     __syncthreads();
     // S = exp(L_end) S + KW^T V
     const float shrink = expf(L_end);
-    const int nt = Np / 4;
+    const int nt = Np / 16;
     const bool state_needed = sp.mode != SPAN_OUTPUTS || c0 + C < n;  // (a span's outputs: nobody reads the state after its last chunk)
-    for (int tile = tid; state_needed && tile < nt * pt; tile += 256) {
-      const int i0 = (tile / pt) * 4, p0 = (tile % pt) * 4;
-      float acc[4][4] = {};
-      for (int j = 0; j < m; ++j) {
-        const float4 kv = *(const float4*)(KW + (size_t)j * Np + i0);
-        const float4 vv = *(const float4*)(V + (size_t)j * Pp + p0);
-        const float ks[4] = {kv.x, kv.y, kv.z, kv.w}, vs[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-#pragma unroll
-          for (int y = 0; y < 4; ++y) acc[x][y] += ks[x] * vs[y];
-      }
+    for (int tile = wave; state_needed && tile < nt * pt; tile += 4) {
+      const int i0 = (tile / pt) * 16, p0 = (tile % pt) * 16;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      const int j_end = (m + 3) & ~3;  // (KW and V are zero from m on)
+      for (int j = 0; j < j_end; j += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(KW[(size_t)(j + lg) * Np + i0 + lr], V[(size_t)(j + lg) * Pp + p0 + lr], acc, 0, 0, 0);
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        float4* sp = (float4*)(S + (size_t)(i0 + x) * Pp + p0);
-        float4 sv = *sp;
-        sv.x = shrink * sv.x + acc[x][0], sv.y = shrink * sv.y + acc[x][1];
-        sv.z = shrink * sv.z + acc[x][2], sv.w = shrink * sv.w + acc[x][3];
-        *sp = sv;
+        float* sp_ = S + (size_t)(i0 + 4 * lg + x) * Pp + p0 + lr;
+        *sp_ = shrink * *sp_ + acc[x];
       }
     }
     // the rows on their way out: a wave a token
@@ -339,22 +305,31 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
   if (sp.mode == SPAN_STATES && tid == 0) sp.span_decay[(size_t)blockIdx.y * a.H + h] = expf(span_log);
 }
 
-// Block (head, request), a thread an element of the state: span_state[s] becomes the state ahead
-// of span s, and the request's row its state after the last span.
+// Block (head, request, 256 elements of the state), a thread an element: span_state[s] becomes
+// the state ahead of span s, and the request's row its state after the last span.  Four spans'
+// values are asked for before the first is used.
 __global__ __launch_bounds__(256) void span_states_kernel(ScanArgs a, SpanArgs sp, const int* __restrict__ span_first) {
-  const int h = blockIdx.x, r = blockIdx.y, NP = a.N * a.P;
+  const int h = blockIdx.x, r = blockIdx.y, NP = a.N * a.P, i = blockIdx.z * 256 + threadIdx.x;
+  if (i >= NP) return;
   const int first = span_first[r], n_spans = (a.seq_len[r] + sp.span - 1) / sp.span;
   float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * NP;
-  for (int i = threadIdx.x; i < NP; i += 256) {
-    float s = Sg[i];
-    for (int c = 0; c < n_spans; ++c) {
-      float* own = sp.span_state + ((size_t)(first + c) * a.H + h) * NP + i;
-      const float add = *own;
-      *own = s;
-      s = sp.span_decay[(size_t)(first + c) * a.H + h] * s + add;
+  float s = Sg[i];
+  for (int c0 = 0; c0 < n_spans; c0 += 4) {
+    float add[4], dec[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = min(c0 + u, n_spans - 1);
+      add[u] = sp.span_state[((size_t)(first + c) * a.H + h) * NP + i];
+      dec[u] = sp.span_decay[(size_t)(first + c) * a.H + h];
     }
-    Sg[i] = s;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c0 + u >= n_spans) break;
+      sp.span_state[((size_t)(first + c0 + u) * a.H + h) * NP + i] = s;
+      s = dec[u] * s + add[u];
+    }
   }
+  Sg[i] = s;
 }
 
 // Queries and keys turned in place ahead of the kernels that take chunks (which would otherwise
@@ -449,7 +424,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 // Floats of LDS that the chunked kernel needs for chunks of C tokens.
 static size_t chunk_floats(int N, int P, int C) {
-  const size_t Np = (N + 3) & ~3, Pp = (P + 3) & ~3, CP = C + 4;
+  const size_t Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
   return 2 * Np * CP + (size_t)C * Np + 2 * (size_t)C * Pp + (size_t)C * CP + Np * Pp;
 }
 
@@ -519,7 +494,7 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
       dim3 span_grid(a.H, n_spans);
       sp = SpanArgs{SPAN_STATES, span, span_req, span_start, span_state, span_decay};
       CHUNKS(span_grid);
-      hipLaunchKernelGGL(span_states_kernel, grid, block, 0, stream, turned, sp, span_first);
+      hipLaunchKernelGGL(span_states_kernel, dim3(a.H, a.n_requests, (a.N * a.P + 255) / 256), block, 0, stream, turned, sp, span_first);
       sp.mode = SPAN_OUTPUTS;
       CHUNKS(span_grid);
     } else {
