@@ -153,7 +153,7 @@ struct SpanArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, SpanArgs sp) {
   extern __shared__ float lds[];
-  __shared__ float Lc[64], Lraw[64];
+  __shared__ float Lc[64], Lraw[64], Ksc[64], Rs[64];
   const int N = a.N, P = a.P, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int Np = (N + 15) & ~15, Pp = (P + 15) & ~15, CP = C + 4;
   const int h = blockIdx.x, hk = h / (a.H / a.Hk);
@@ -174,45 +174,59 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
     const int kn = i / Pp, p = i % Pp;
     S[i] = sp.mode != SPAN_STATES && kn < N && p < P ? Sg[(size_t)kn * P + p] : 0.f;
   }
-  const int half = a.rot_dims / 2;
   const float log_decay = a.log_a ? 0.f : logf(a.decay[h]);
   const bool outputs = sp.mode != SPAN_STATES;
   float span_log = 0.f;
   for (int c0 = lo; c0 < n; c0 += C) {
     const int m = min(C, n - c0);
     const size_t row0 = (size_t)(start + c0);
+    // (Lraw and Ksc are read only ahead of the chunk's second barrier, so the chunk before is done with them)
+    if (tid < C) {
+      const size_t rt = (row0 + min(tid, m - 1)) * a.H + h;
+      Lraw[tid] = tid < m ? (a.log_a ? a.log_a[rt] : log_decay) : 0.f;
+      Ksc[tid] = a.k_mult * (a.k_scale ? a.k_scale[rt] : 1.0f);
+    }
     __syncthreads();  // the chunk before is done with every array (and S is loaded)
-    if (tid < C) Lraw[tid] = tid < m ? (a.log_a ? a.log_a[(row0 + tid) * a.H + h] : log_decay) : 0.f;
-    // queries and keys, turned and scaled, transposed; a pair of turning columns is one item
-    const int items = N - half;  // pairs (i, i + half) for i < half, then the columns from rot_dims on
-    for (int e = tid; e < C * items; e += 256) {
-      const int t = e / items, it = e % items;
-      float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
-      const int i = it < half ? it : it + half;
-      if (t < m) {
-        const float* qr = a.q + (row0 + t) * a.ldq + (size_t)hk * N;
-        const float* kr = a.k + (row0 + t) * a.ldk + (size_t)hk * N;
-        const float ksc = a.k_mult * (a.k_scale ? a.k_scale[(row0 + t) * a.H + h] : 1.0f);
-        if (it < half) {
-          float sn, cs;
-          sincosf((float)a.positions[row0 + t] * a.inv_freq[it], &sn, &cs);
-          const float qa = qr[it], qb = qr[it + half], ka = kr[it], kb = kr[it + half];
-          q0 = qa * cs - qb * sn, q1 = qb * cs + qa * sn;
-          k0 = (ka * cs - kb * sn) * ksc, k1 = (kb * cs + ka * sn) * ksc;
-        } else {
-          q0 = qr[i], k0 = kr[i] * ksc;
+    // Queries and keys (turned already, see the launcher), scaled keys, transposed; values.  Eight
+    // loads a thread are asked for before the first is stored; addresses are pulled inside the
+    // chunk and what lies outside is zeroed afterwards.
+    {
+      const int total = C * N;
+      const float* qb = a.q + row0 * a.ldq + (size_t)hk * N;
+      const float* kb = a.k + row0 * a.ldk + (size_t)hk * N;
+      for (int base = 0; base < total; base += 256 * 8) {
+        float qv[8], kv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int e = min(base + u * 256 + tid, total - 1), t = e / N, i = e - t * N, tc = min(t, m - 1);
+          qv[u] = qb[(size_t)tc * a.ldq + i], kv[u] = kb[(size_t)tc * a.ldk + i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int e = base + u * 256 + tid, t = e / N, i = e - t * N;
+          if (e < total) QT[(size_t)i * CP + t] = t < m ? qv[u] : 0.f, KT[(size_t)i * CP + t] = t < m ? kv[u] * Ksc[t] : 0.f;
         }
       }
-      QT[(size_t)i * CP + t] = q0, KT[(size_t)i * CP + t] = k0;
-      if (it < half) QT[(size_t)(it + half) * CP + t] = q1, KT[(size_t)(it + half) * CP + t] = k1;
-    }
-    for (int e = tid; e < C * (Np - N); e += 256) {  // the padding
-      const int t = e / (Np - N), i = N + e % (Np - N);
-      QT[(size_t)i * CP + t] = 0.f, KT[(size_t)i * CP + t] = 0.f;
-    }
-    for (int e = tid; e < C * Pp; e += 256) {
-      const int t = e / Pp, p = e % Pp;
-      V[e] = t < m && p < P ? a.v[(row0 + t) * a.ldv + (size_t)h * P + p] : 0.f;
+      for (int e = tid; e < C * (Np - N); e += 256) {  // the padding
+        const int t = e / (Np - N), i = N + e % (Np - N);
+        QT[(size_t)i * CP + t] = 0.f, KT[(size_t)i * CP + t] = 0.f;
+      }
+      const int v_total = C * P;
+      const float* vb = a.v + row0 * a.ldv + (size_t)h * P;
+      for (int base = 0; base < v_total; base += 256 * 8) {
+        float vv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int e = min(base + u * 256 + tid, v_total - 1), t = e / P, pc = e - t * P;
+          vv[u] = vb[(size_t)min(t, m - 1) * a.ldv + pc];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int e = base + u * 256 + tid, t = e / P, pc = e - t * P;
+          if (e < v_total) V[(size_t)t * Pp + pc] = t < m ? vv[u] : 0.f;
+        }
+      }
+      for (int e = tid; e < C * (Pp - P); e += 256) V[(size_t)(e / (Pp - P)) * Pp + P + e % (Pp - P)] = 0.f;
     }
     __syncthreads();
     if (tid < C) {
@@ -284,18 +298,31 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
         *sp_ = shrink * *sp_ + acc[x];
       }
     }
-    // the rows on their way out: a wave a token
-    for (int t = wave; outputs && t < m; t += 4) {
-      float rstd = 1.f;
-      if (a.unit_rms) {
+    // the rows on their way out: a wave a token; the gates of eight tokens are asked for at once
+    if (outputs && a.unit_rms)
+      for (int t = wave; t < m; t += 4) {
         float ss = 0.f;
-        for (int p = lane; p < P; p += 64) ss += O[(size_t)t * Pp + p] * O[(size_t)t * Pp + p];
-        rstd = 1.0f / sqrtf(wave_sum(ss) / (float)P + a.eps);
+        for (int pc = lane; pc < P; pc += 64) ss += O[(size_t)t * Pp + pc] * O[(size_t)t * Pp + pc];
+        ss = wave_sum(ss);
+        if (lane == 0) Rs[t] = 1.0f / sqrtf(ss / (float)P + a.eps);
       }
-      for (int p = lane; p < P; p += 64) {
-        float o = O[(size_t)t * Pp + p] * rstd;
-        if (a.gate) o *= silu_f(a.gate[(row0 + t) * a.ldg + (size_t)h * P + p]);
-        ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + p] = from_f32<T>(o);
+    // (a wave reads the Rs it wrote itself: tokens wave, wave + 4, ...)
+    for (int pb = 0; outputs && pb < P; pb += 64) {
+      const int pc = min(pb + lane, P - 1);
+      for (int tb = wave; tb < m; tb += 32) {
+        float gv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          gv[u] = a.gate ? a.gate[(row0 + min(tb + 4 * u, m - 1)) * a.ldg + (size_t)h * P + pc] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int t = tb + 4 * u;
+          if (t >= m || pb + lane >= P) continue;
+          float o = O[(size_t)t * Pp + pc];
+          if (a.unit_rms) o *= Rs[t];
+          if (a.gate) o *= silu_f(gv[u]);
+          ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + pc] = from_f32<T>(o);
+        }
       }
     }
   }
@@ -464,7 +491,7 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
     for (int c = 64; c >= 16 && !C; c /= 2)
       if (chunk_floats(a.N, a.P, c) * sizeof(float) <= SCAN_MAX_LDS) C = c;
   if (C) {
-    ScanArgs turned = a;
+    ScanArgs turned = a;  // (the chunked kernel itself turns nothing)
     if (a.rot_dims) {
       // (q and k are the caller's work memory: the projection's rows, which nothing reads after this)
       const long items = (long)a.n_tokens_hint * a.Hk * (a.rot_dims / 2);
