@@ -69,7 +69,14 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
   float* partial = vs + P;  // [parts, P]
   const int start = a.seq_start[r], n = a.seq_len[r];
   float* Sg = a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P;
-  for (int i = tid; i < N * P; i += 256) S[i] = Sg[i];
+  for (int base = 0; base < N * P; base += 256 * 8) {  // (eight loads a thread on their way at once)
+    float sv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sv[u] = Sg[min(base + u * 256 + tid, N * P - 1)];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (base + u * 256 + tid < N * P) S[base + u * 256 + tid] = sv[u];
+  }
   const int half = a.rot_dims / 2;
   const int p = tid % P, part = tid / P;
   const bool works = tid < parts * P;

@@ -140,16 +140,17 @@ def _ints(values):
 # -- each mechanism's kernels alone -------------------------------------------------------
 
 
-@pytest.mark.parametrize("width", [64, 100, 1000])
+@pytest.mark.parametrize("width,rows", [(64, 7), (100, 7), (1000, 7), (1000, 70), (2500, 3), (300, 65)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_the_sum_between_two_norms(width, dtype):
+def test_the_sum_between_two_norms(width, rows, dtype):
+    """Few rows: a wave a row with the row in registers; many rows or wide ones: a block a row."""
     from mlx_lm_amd.ops import kernels
 
     g = torch.Generator().manual_seed(width)
-    h, y = (torch.randn(7, width, generator=g) * 3).cuda(), (torch.randn(7, width, generator=g) * 5 + 1).cuda()
+    h, y = (torch.randn(rows, width, generator=g) * 3).cuda(), (torch.randn(rows, width, generator=g) * 5 + 1).cuda()
     w1, w2 = (1 + 0.3 * torch.randn(width, generator=g)).cuda(), (1 + 0.3 * torch.randn(width, generator=g)).cuda()
     want_h = h.double().cpu() + 0.7 * plain.layer_norm(y.double().cpu(), w1.double().cpu(), 1e-3)
-    out = torch.empty(7, width, dtype=dtype, device="cuda")
+    out = torch.empty(rows, width, dtype=dtype, device="cuda")
     h1, h2 = h.clone(), h.clone()
     kernels.add_normed(h1, y, w1, 0.7, 1e-3)
     kernels.add_normed(h2, y, w1, 0.7, 1e-3, w2, out)
