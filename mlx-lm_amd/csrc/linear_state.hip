@@ -454,7 +454,7 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* _
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-#define SCAN_MAX_LDS (152 * 1024)
+#define SCAN_MAX_LDS (158 * 1024)
 
 // Floats of LDS that the chunked kernel needs for chunks of C tokens.
 static size_t chunk_floats(int N, int P, int C) {
