@@ -42,6 +42,23 @@ def _matrix(w):
     return kernels.for_decode(w.contiguous())
 
 
+def _padded_columns(w, multiple=8):
+    """``w`` ``[N, K]`` with zero columns up to the next multiple of ``multiple`` (what a product's
+    inner size has to be); the rows that meet them carry zeros in those columns."""
+    pad = -w.shape[1] % multiple
+    return torch.cat([w, w.new_zeros(w.shape[0], pad)], 1) if pad else w
+
+
+def _rows_for(ctx, n_rows, width, padded):
+    """Rows of ``width`` columns for a product whose inner size is ``padded``: a view of zeroed wider
+    rows where the two differ."""
+    if padded == width:
+        return ctx.scratch((n_rows, width), ctx.dtype), None
+    whole = ctx.scratch((n_rows, padded), ctx.dtype)
+    whole.zero_()
+    return whole[:, :width], whole
+
+
 class Retention(_SequenceArrays, Mixer):
     """Linear attention with a fixed decay per head and neither softmax nor denominator:
 
@@ -70,8 +87,8 @@ class Retention(_SequenceArrays, Mixer):
             raise ValueError(f"{len(decay)} decays for {n_heads} heads")
         if rot_dims % 2 or not 0 <= rot_dims <= key_dim:
             raise ValueError(f"{rot_dims} turning columns of {key_dim}: an even number within the head")
-        if width % 8 or (n_heads * value_dim) % 8:
-            raise ValueError(f"width {width} and the heads' value columns {n_heads * value_dim} must be multiples of 8")
+        if width % 8:
+            raise ValueError(f"width {width} must be a multiple of 8")
         self.width, self.n_heads, self.key_dim, self.value_dim = width, n_heads, key_dim, value_dim
         self.decay_values, self.eps = [float(d) for d in decay], float(eps)
         self.rot_dims, self.rot_base = int(rot_dims), float(rot_base)
@@ -96,7 +113,7 @@ class Retention(_SequenceArrays, Mixer):
         n = self.names
         dev = tensors[n["q"]].device
         self.in_w = _matrix(torch.cat([tensors[n[x]] for x in ("q", "k", "v", "g")]))
-        self.out_w = _matrix(tensors[n["o"]])
+        self.out_w = _matrix(_padded_columns(tensors[n["o"]]))
         self.first_weight = self.in_w
         self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=dev)
         half = self.rot_dims // 2
@@ -110,14 +127,14 @@ class Retention(_SequenceArrays, Mixer):
         u = ctx.scratch((T, 2 * self.qk_width + 2 * self.v_width), torch.float32)
         kernels.linear(u, x, self.in_w)
         a, b = self.qk_width, 2 * self.qk_width
-        out = ctx.scratch((T, self.v_width), ctx.dtype)
+        out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
         kernels.state_scan(out, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, 0,
                            ctx.array("sequences.starts"), ctx.array("sequences.lens"), ctx.slot_ids, ctx.n_requests,
                            self.n_heads, self.n_heads, self.key_dim, self.value_dim, decay=self.decay,
                            k_mult=self.key_scale, rot_dims=self.rot_dims, inv_freq=self.inv_freq,
                            positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:],
                            chunked=self._chunked(ctx), spans=self._spans(ctx))
-        kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite)
         ctx.scratch_release(mark)
 
 
@@ -150,8 +167,8 @@ class StateSpace(_SequenceArrays, Mixer):
         inner = n_heads * value_dim
         if norm_groups <= 0 or inner % norm_groups:
             raise ValueError(f"{inner} inner columns cannot be normed in {norm_groups} equal parts")
-        if width % 8 or inner % 8:
-            raise ValueError(f"width {width} and the inner size {inner} must be multiples of 8")
+        if width % 8:
+            raise ValueError(f"width {width} must be a multiple of 8")
         self.width, self.n_heads, self.value_dim, self.state, self.groups = width, n_heads, value_dim, state, groups
         self.taps, self.norm_groups, self.eps, self.inner = int(taps), int(norm_groups), float(eps), inner
         self.channels = inner + 2 * groups * state
@@ -177,7 +194,7 @@ class StateSpace(_SequenceArrays, Mixer):
 
     def load(self, tensors):
         n = self.names
-        self.in_w, self.out_w = _matrix(tensors[n["in"]]), _matrix(tensors[n["o"]])
+        self.in_w, self.out_w = _matrix(tensors[n["in"]]), _matrix(_padded_columns(tensors[n["o"]]))
         self.first_weight = self.in_w
         self.conv_w, self.conv_b = tensors[n["conv"]].contiguous(), tensors[n["conv.b"]]
         self.dt_bias, self.a_log, self.skip = tensors[n["dt_bias"]], tensors[n["A_log"]], tensors[n["D"]]
@@ -201,9 +218,9 @@ class StateSpace(_SequenceArrays, Mixer):
                            cache.state, self.conv_floats, starts, lens, ctx.slot_ids, ctx.n_requests, H, self.groups,
                            self.state, self.value_dim, log_a=log_a, k_scale=dt, skip=self.skip, chunked=self._chunked(ctx),
                            spans=self._spans(ctx))
-        out = ctx.scratch((T, self.inner), ctx.dtype)
+        out, whole = _rows_for(ctx, T, self.inner, -(-self.inner // 8) * 8)
         kernels.gated_group_rmsnorm(out, y, u[:, :self.inner], self.norm_w, self.norm_groups, self.eps)
-        kernels.linear(residual, out, self.out_w, accumulate=not self.overwrite)
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite)
         ctx.scratch_release(mark)
 
 

@@ -544,7 +544,9 @@ def test_twenty_requests_decode_together(models, dtype):
 
 def test_models_without_pages_and_without_state(tmp_path):
     """Only retention layers (no cache group at all), and only a parallel layer without a window."""
-    for name, layers in (("r", [_moe(_retention(2, 16, 16, [0.9, 0.99], rot_dims=8), 3, 1, 2, 16), _retention(1, 8, 24, [0.7])]),
+    # (also: value columns and an inner size that are no multiples of 8, whose output products get zero columns)
+    for name, layers in (("r", [_moe(_retention(2, 16, 16, [0.9, 0.99], rot_dims=8), 3, 1, 2, 16), _retention(1, 8, 24, [0.7]),
+                                _retention(3, 6, 20, [0.8, 0.9, 0.95], rot_dims=6), _parallel(1, 1, 8, 8, 5, 3, 4, 6, 3, 2, 1)]),
                          ("p", [_moe(_parallel(2, 1, 16, 16, None, 2, 8, 8, 1, 3, 1), 2, 0, 1, 8)])):
         config = _config(48, 61, layers, mult=0.9)
         weights = plain.random_weights(config, 12, sharp=2.0)
