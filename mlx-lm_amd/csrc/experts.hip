@@ -225,10 +225,11 @@ struct Frag<float> {
   }
 };
 
-// Block (tile, 256 features): a wave all of the tile's picks (four groups of 16) x 64 features of
-// gate and of up, operands straight from memory; a weight fragment meets up to four fragments of
-// rows.  act[pick, f] = weight * silu(gate) * up.
-template <typename T>
+// Block (tile, 64 CF features): a wave all of the tile's picks (four groups of 16) x 16 CF features
+// of gate and of up, operands straight from memory; a weight fragment meets up to four fragments
+// of rows.  CF = 4 where the tiles alone fill the GPU, 1 where they are few (a decode step of some
+// dozen tokens), so that the blocks are four times as many.  act[pick, f] = weight * silu(gate) * up.
+template <typename T, int CF>
 __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w_gate,
                                                               const T* __restrict__ w_up, const int* __restrict__ order,
                                                               const int* __restrict__ tiles, const int* __restrict__ n_tiles,
@@ -238,40 +239,40 @@ __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restric
   if ((int)blockIdx.x >= *n_tiles) return;
   const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
-  const int f0 = blockIdx.y * 256 + wave * 64;
+  const int f0 = (blockIdx.y * 4 + wave) * 16 * CF;
   if (f0 >= F) return;  // (no barrier in this kernel)
   const int groups = (count + 15) / 16;
   const T* xrow[4];
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg) xrow[rg] = x + (size_t)(order[first + min(16 * rg + r, count - 1)] / top) * ldx;
-  const T* grow[4];
-  const T* urow[4];
+  const T* grow[CF];
+  const T* urow[CF];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int c = 0; c < CF; ++c) {
     const size_t f = (size_t)e * F + min(f0 + 16 * c + r, F - 1);
     grow[c] = w_gate + f * width, urow[c] = w_up + f * width;
   }
-  f32x4_t ag[4][4], au[4][4];
+  f32x4_t ag[4][CF], au[4][CF];
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
-    for (int c = 0; c < 4; ++c) ag[rg][c] = au[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < CF; ++c) ag[rg][c] = au[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   // two sets of operands by turns: the next step's loads are on their way during this step's products
   // (the width is a multiple of KL: a lane's values are all inside or all outside)
-  typename Fr::V a[2][4], bg[2][4], bu[2][4];
+  typename Fr::V a[2][4], bg[2][CF], bu[2][CF];
   const int step = 4 * Fr::KL;
 #define LOAD_SET(S, K0)                                                                                 \
   do {                                                                                                  \
     const int k_ = (K0) + Fr::KL * g;                                                                   \
     const bool in_ = k_ < width;                                                                        \
     _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) a[S][rg] = Fr::load(xrow[rg] + k_, in_);           \
-    _Pragma("unroll") for (int c = 0; c < 4; ++c) bg[S][c] = Fr::load(grow[c] + k_, in_), bu[S][c] = Fr::load(urow[c] + k_, in_); \
+    _Pragma("unroll") for (int c = 0; c < CF; ++c) bg[S][c] = Fr::load(grow[c] + k_, in_), bu[S][c] = Fr::load(urow[c] + k_, in_); \
   } while (0)
 #define MMA_SET(S)                                                                                      \
   do {                                                                                                  \
     _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) {                                                  \
       if (rg < groups) { /* (the same for every lane of the block) */                                   \
-        _Pragma("unroll") for (int c = 0; c < 4; ++c) {                                                 \
+        _Pragma("unroll") for (int c = 0; c < CF; ++c) {                                                 \
           ag[rg][c] = Fr::mma(a[S][rg], bg[S][c], ag[rg][c]);                                           \
           au[rg][c] = Fr::mma(a[S][rg], bu[S][c], au[rg][c]);                                           \
         }                                                                                               \
@@ -296,15 +297,15 @@ __global__ __launch_bounds__(256) void expert_tiles_up_kernel(const T* __restric
       const int it = order[first + ri];
       const float wt = weight[it];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
+      for (int c = 0; c < CF; ++c) {
         const int f = f0 + 16 * c + r;
         if (f < F) act[(size_t)it * F + f] = from_f32<T>(wt * silu_f(ag[rg][c][i]) * au[rg][c][i]);
       }
     }
 }
 
-// Block (tile, 256 columns): out[pick, n] = sum_f act[pick, f] w_down[e, n, f], laid out as above.
-template <typename T>
+// Block (tile, 64 CF columns): out[pick, n] = sum_f act[pick, f] w_down[e, n, f], laid out as above.
+template <typename T, int CF>
 __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
                                                                 const int* __restrict__ order, const int* __restrict__ tiles,
                                                                 const int* __restrict__ n_tiles, int F, int width,
@@ -313,34 +314,34 @@ __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restr
   if ((int)blockIdx.x >= *n_tiles) return;
   const int e = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], count = tiles[3 * blockIdx.x + 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, r = lane & 15;
-  const int n0 = blockIdx.y * 256 + wave * 64;
+  const int n0 = (blockIdx.y * 4 + wave) * 16 * CF;
   if (n0 >= width) return;
   const int groups = (count + 15) / 16;
   const T* arow[4];
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg) arow[rg] = act + (size_t)order[first + min(16 * rg + r, count - 1)] * F;
-  const T* drow[4];
+  const T* drow[CF];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) drow[c] = w_down + ((size_t)e * width + min(n0 + 16 * c + r, width - 1)) * F;
-  f32x4_t acc[4][4];
+  for (int c = 0; c < CF; ++c) drow[c] = w_down + ((size_t)e * width + min(n0 + 16 * c + r, width - 1)) * F;
+  f32x4_t acc[4][CF];
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg)
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  typename Fr::V a[2][4], b[2][4];
+    for (int c = 0; c < CF; ++c) acc[rg][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  typename Fr::V a[2][4], b[2][CF];
   const int step = 4 * Fr::KL;
 #define LOAD_SET(S, K0)                                                                        \
   do {                                                                                         \
     const int k_ = (K0) + Fr::KL * g;                                                          \
     const bool in_ = k_ < F;                                                                   \
     _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) a[S][rg] = Fr::load(arow[rg] + k_, in_);  \
-    _Pragma("unroll") for (int c = 0; c < 4; ++c) b[S][c] = Fr::load(drow[c] + k_, in_);       \
+    _Pragma("unroll") for (int c = 0; c < CF; ++c) b[S][c] = Fr::load(drow[c] + k_, in_);       \
   } while (0)
 #define MMA_SET(S)                                                                             \
   do {                                                                                         \
     _Pragma("unroll") for (int rg = 0; rg < 4; ++rg) {                                         \
       if (rg < groups) {                                                                       \
-        _Pragma("unroll") for (int c = 0; c < 4; ++c) acc[rg][c] = Fr::mma(a[S][rg], b[S][c], acc[rg][c]); \
+        _Pragma("unroll") for (int c = 0; c < CF; ++c) acc[rg][c] = Fr::mma(a[S][rg], b[S][c], acc[rg][c]); \
       }                                                                                        \
     }                                                                                          \
   } while (0)
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(256) void expert_tiles_down_kernel(const T* __restr
       if (ri >= count) continue;
       const size_t it = order[first + ri];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
+      for (int c = 0; c < CF; ++c) {
         const int n = n0 + 16 * c + r;
         if (n < width) out[it * width + n] = acc[rg][c][i];
       }
@@ -474,20 +475,24 @@ extern "C" int expert_tiles(const void* x, int ldx, const void* w_gate, const vo
   const int n_items = n_tokens * top, most = expert_tiles_most(n_items, n_experts);
   hipLaunchKernelGGL(expert_sort_kernel, dim3(1), dim3(1024), 2 * n_experts * sizeof(int), stream, idx, n_items, n_experts,
                      order, tiles, n_tiles);
-  dim3 block(256), up_grid(most, (F + 255) / 256), down_grid(most, (width + 255) / 256), sum_grid(n_tokens, (width + 255) / 256);
-#define RUN(T)                                                                                                          \
-  do {                                                                                                                  \
-    hipLaunchKernelGGL(expert_tiles_up_kernel<T>, up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,        \
-                       (const T*)w_up, order, tiles, n_tiles, weight, top, F, width, (T*)act);                          \
-    hipLaunchKernelGGL(expert_tiles_down_kernel<T>, down_grid, block, 0, stream, (const T*)act, (const T*)w_down, order, \
-                       tiles, n_tiles, F, width, out);                                                                  \
-    hipLaunchKernelGGL(expert_combine_kernel<T>, sum_grid, block, 0, stream, out, idx, weight, (const T*)x, ldx,        \
-                       n_experts, top, width, y, ldy, accumulate);                                                      \
+  // (wide blocks where the tiles alone fill the GPU, narrow ones where they are few)
+  const bool wide = (long)most * ((F + 255) / 256) >= 256;
+  const int per = wide ? 256 : 64;
+  dim3 block(256), up_grid(most, (F + per - 1) / per), down_grid(most, (width + per - 1) / per), sum_grid(n_tokens, (width + 255) / 256);
+#define RUN(T, CF)                                                                                                       \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL((expert_tiles_up_kernel<T, CF>), up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,   \
+                       (const T*)w_up, order, tiles, n_tiles, weight, top, F, width, (T*)act);                           \
+    hipLaunchKernelGGL((expert_tiles_down_kernel<T, CF>), down_grid, block, 0, stream, (const T*)act, (const T*)w_down,  \
+                       order, tiles, n_tiles, F, width, out);                                                            \
+    hipLaunchKernelGGL(expert_combine_kernel<T>, sum_grid, block, 0, stream, out, idx, weight, (const T*)x, ldx,         \
+                       n_experts, top, width, y, ldy, accumulate);                                                       \
   } while (0)
-  if (dtype == DT_F32)
-    RUN(float);
-  else
-    RUN(bf16);
+  if (dtype == DT_F32) {
+    if (wide) RUN(float, 4); else RUN(float, 1);
+  } else {
+    if (wide) RUN(bf16, 4); else RUN(bf16, 1);
+  }
 #undef RUN
   CHECK_LAUNCH("expert_tiles");
   return 0;

@@ -302,6 +302,14 @@ SPLIT_WS_FLOATS = 8 << 20  # 32 MB: sixteen splits of 64 rows by 8192 features
 force_splits = 0
 
 
+def splits_alone(n_rows):
+    """``splits`` for a product of ``n_rows`` rows whose partial sums nobody else would add (a part
+    written in Python has no norm behind it that takes them): 17 to 64 rows go unsplit, since the
+    second kernel that adds the parts costs more there than the split saves (a decode step of 32
+    rows, 1,024 wide: 1.92 ms against 2.08); otherwise the library chooses."""
+    return 1 if DECODE_MAX_ROWS < n_rows <= 64 else None
+
+
 def split_workspace(device):
     """Float32 room for the partial sums of projections that split K over blocks.
 

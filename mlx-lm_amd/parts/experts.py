@@ -29,7 +29,7 @@ class GatedExperts(FeedForward):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     can_overwrite = True
-    TILES_FROM = 128  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
+    TILES_FROM = 64  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
 
     def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, prefix=""):
         super().__init__(prefix)
@@ -87,17 +87,17 @@ class GatedExperts(FeedForward):
         T = x.shape[0]
         mark = ctx.scratch_mark()
         z = ctx.scratch((T, self.n_out), torch.float32)
-        kernels.linear(z, x, self.router_w)
+        kernels.linear(z, x, self.router_w, splits=kernels.splits_alone(T))
         idx = ctx.scratch((T, self.top), torch.int32)
         weight = ctx.scratch((T, self.top), torch.float32)
         kernels.router_choice(idx, weight, z, self.correction, self.top)
         accumulate = not self.overwrite
         if self.shared_inner:
             gu = ctx.scratch((T, 2 * self.shared_padded), ctx.dtype)
-            kernels.linear(gu, x, self.shared_in)
+            kernels.linear(gu, x, self.shared_in, splits=kernels.splits_alone(T))
             act = ctx.scratch((T, self.shared_padded), ctx.dtype)
             kernels.silu_mul(act, gu)
-            kernels.linear(residual, act, self.shared_out, accumulate=accumulate)
+            kernels.linear(residual, act, self.shared_out, accumulate=accumulate, splits=kernels.splits_alone(T))
             accumulate = True
         if self.n_experts and T >= self.TILES_FROM and kernels.expert_tiles_takes(self.inner, self.width, x.dtype):
             kernels.expert_tiles(residual, x, self.w_gate, self.w_up, self.w_down, idx, weight, self.top, ctx.scratch,

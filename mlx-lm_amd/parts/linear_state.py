@@ -125,7 +125,7 @@ class Retention(_SequenceArrays, Mixer):
         T = x.shape[0]
         mark = ctx.scratch_mark()
         u = ctx.scratch((T, 2 * self.qk_width + 2 * self.v_width), torch.float32)
-        kernels.linear(u, x, self.in_w)
+        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
         a, b = self.qk_width, 2 * self.qk_width
         out, whole = _rows_for(ctx, T, self.v_width, -(-self.v_width // 8) * 8)
         kernels.state_scan(out, u[:, :a], u[:, a:b], u[:, b:b + self.v_width], cache.state, 0,
@@ -134,7 +134,7 @@ class Retention(_SequenceArrays, Mixer):
                            k_mult=self.key_scale, rot_dims=self.rot_dims, inv_freq=self.inv_freq,
                            positions=ctx.positions, unit_rms=True, eps=self.eps, gate=u[:, b + self.v_width:],
                            chunked=self._chunked(ctx), spans=self._spans(ctx))
-        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite)
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite, splits=kernels.splits_alone(T))
         ctx.scratch_release(mark)
 
 
@@ -204,7 +204,7 @@ class StateSpace(_SequenceArrays, Mixer):
         T, H, GN = x.shape[0], self.n_heads, self.groups * self.state
         mark = ctx.scratch_mark()
         u = ctx.scratch((T, self.in_width), torch.float32)
-        kernels.linear(u, x, self.in_w)
+        kernels.linear(u, x, self.in_w, splits=kernels.splits_alone(T))
         xbc = ctx.scratch((T, self.channels), torch.float32)
         dt = ctx.scratch((T, H), torch.float32)
         log_a = ctx.scratch((T, H), torch.float32)
@@ -220,7 +220,7 @@ class StateSpace(_SequenceArrays, Mixer):
                            spans=self._spans(ctx))
         out, whole = _rows_for(ctx, T, self.inner, -(-self.inner // 8) * 8)
         kernels.gated_group_rmsnorm(out, y, u[:, :self.inner], self.norm_w, self.norm_groups, self.eps)
-        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite)
+        kernels.linear(residual, out if whole is None else whole, self.out_w, accumulate=not self.overwrite, splits=kernels.splits_alone(T))
         ctx.scratch_release(mark)
 
 
