@@ -177,9 +177,18 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
   const int n = sp.mode == WHOLE ? a.seq_len[r] : min(a.seq_len[r], lo + sp.span);
   float* Sg = sp.mode == WHOLE ? a.state + (size_t)a.slot_ids[r] * a.state_stride + a.state_offset + (size_t)h * N * P
                                : sp.span_state + ((size_t)blockIdx.y * a.H + h) * N * P;
-  for (int i = tid; i < Np * Pp; i += 256) {
-    const int kn = i / Pp, p = i % Pp;
-    S[i] = sp.mode != SPAN_STATES && kn < N && p < P ? Sg[(size_t)kn * P + p] : 0.f;
+  for (int base = 0; base < Np * Pp; base += 256 * 8) {  // (eight loads a thread on their way at once)
+    float sv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = min(base + u * 256 + tid, Np * Pp - 1), kn = min(i / Pp, N - 1), p = min(i % Pp, P - 1);
+      sv[u] = sp.mode != SPAN_STATES ? Sg[(size_t)kn * P + p] : 0.f;  // (the same for every thread: no lane waits for another's load)
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = base + u * 256 + tid;
+      if (i < Np * Pp) S[i] = i / Pp < N && i % Pp < P ? sv[u] : 0.f;
+    }
   }
   const float log_decay = a.log_a ? 0.f : logf(a.decay[h]);
   const bool outputs = sp.mode != SPAN_STATES;
@@ -187,51 +196,57 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
   for (int c0 = lo; c0 < n; c0 += C) {
     const int m = min(C, n - c0);
     const size_t row0 = (size_t)(start + c0);
-    // (Lraw and Ksc are read only ahead of the chunk's second barrier, so the chunk before is done with them)
+    // Everything the chunk reads from memory is asked for at once, ahead of the barrier: a token's
+    // decay and key scale (thread t < C), queries, keys (turned already, see the launcher) and
+    // values sixteen a thread, and the gates that the rows meet on their way out.  Addresses are
+    // pulled inside the chunk; what lies outside is zeroed when it is stored.  (Trips to memory one
+    // after the other, not the products, are what a chunk's time is made of.)
+    float lraw = 0.f, ksc = 1.f;
     if (tid < C) {
       const size_t rt = (row0 + min(tid, m - 1)) * a.H + h;
-      Lraw[tid] = tid < m ? (a.log_a ? a.log_a[rt] : log_decay) : 0.f;
-      Ksc[tid] = a.k_mult * (a.k_scale ? a.k_scale[rt] : 1.0f);
+      lraw = tid < m ? (a.log_a ? a.log_a[rt] : log_decay) : 0.f;
+      ksc = a.k_mult * (a.k_scale ? a.k_scale[rt] : 1.0f);
     }
-    __syncthreads();  // the chunk before is done with every array (and S is loaded)
-    // Queries and keys (turned already, see the launcher), scaled keys, transposed; values.  Eight
-    // loads a thread are asked for before the first is stored; addresses are pulled inside the
-    // chunk and what lies outside is zeroed afterwards.
+    const bool gates_ahead = outputs && a.gate && P <= 64;
+    float gv[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      gv[u] = gates_ahead ? a.gate[(row0 + min(wave + 4 * u, m - 1)) * a.ldg + (size_t)h * P + min(lane, P - 1)] : 0.f;
     {
-      const int total = C * N;
+      const int total = C * N, v_total = C * P, most = max(total, v_total);
       const float* qb = a.q + row0 * a.ldq + (size_t)hk * N;
       const float* kb = a.k + row0 * a.ldk + (size_t)hk * N;
-      for (int base = 0; base < total; base += 256 * 8) {
-        float qv[8], kv[8];
+      const float* vb = a.v + row0 * a.ldv + (size_t)h * P;
+      bool first = true;
+      for (int base = 0; base < most; base += 256 * 16) {
+        float qv[16], kv[16], vv[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int e = min(base + u * 256 + tid, total - 1), t = e / N, i = e - t * N, tc = min(t, m - 1);
+        for (int u = 0; u < 16; ++u) {
+          const int e = base + u * 256 + tid;
+          const int eq = min(e, total - 1), t = eq / N, i = eq - t * N, tc = min(t, m - 1);
           qv[u] = qb[(size_t)tc * a.ldq + i], kv[u] = kb[(size_t)tc * a.ldk + i];
+          const int ev = min(e, v_total - 1), tv = ev / P;
+          vv[u] = vb[(size_t)min(tv, m - 1) * a.ldv + (ev - tv * P)];
         }
+        if (first) __syncthreads();  // the chunk before is done with every array (and S is loaded)
+        first = false;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int e = base + u * 256 + tid, t = e / N, i = e - t * N;
-          if (e < total) QT[(size_t)i * CP + t] = t < m ? qv[u] : 0.f, KT[(size_t)i * CP + t] = t < m ? kv[u] * Ksc[t] : 0.f;
+        for (int u = 0; u < 16; ++u) {
+          const int e = base + u * 256 + tid;
+          if (e < total) {
+            const int t = e / N, i = e - t * N;
+            QT[(size_t)i * CP + t] = t < m ? qv[u] : 0.f, KT[(size_t)i * CP + t] = t < m ? kv[u] : 0.f;
+          }
+          if (e < v_total) {
+            const int t = e / P;
+            V[(size_t)t * Pp + (e - t * P)] = t < m ? vv[u] : 0.f;
+          }
         }
       }
+      if (tid < C) Lraw[tid] = lraw, Ksc[tid] = ksc;
       for (int e = tid; e < C * (Np - N); e += 256) {  // the padding
         const int t = e / (Np - N), i = N + e % (Np - N);
         QT[(size_t)i * CP + t] = 0.f, KT[(size_t)i * CP + t] = 0.f;
-      }
-      const int v_total = C * P;
-      const float* vb = a.v + row0 * a.ldv + (size_t)h * P;
-      for (int base = 0; base < v_total; base += 256 * 8) {
-        float vv[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int e = min(base + u * 256 + tid, v_total - 1), t = e / P, pc = e - t * P;
-          vv[u] = vb[(size_t)min(t, m - 1) * a.ldv + pc];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int e = base + u * 256 + tid, t = e / P, pc = e - t * P;
-          if (e < v_total) V[(size_t)t * Pp + pc] = t < m ? vv[u] : 0.f;
-        }
       }
       for (int e = tid; e < C * (Pp - P); e += 256) V[(size_t)(e / (Pp - P)) * Pp + P + e % (Pp - P)] = 0.f;
     }
@@ -245,7 +260,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
     const float L_end = Lc[m - 1];
     for (int e = tid; e < C * Np; e += 256) {
       const int j = e / Np, i = e % Np;
-      KW[e] = j < m ? KT[(size_t)i * CP + j] * expf(L_end - Lc[j]) : 0.f;
+      KW[e] = j < m ? KT[(size_t)i * CP + j] * (Ksc[j] * expf(L_end - Lc[j])) : 0.f;
     }
     span_log += L_end;
     // The three products run on the matrix cores in 32-bit (v_mfma_f32_16x16x4_f32: lane l brings
@@ -265,7 +280,7 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
         const int t = t0 + 4 * lg + x;
-        ov[x] = j <= t && t < m ? acc[x] * expf(Lc[t] - Lc[j]) : 0.f;
+        ov[x] = j <= t && t < m ? acc[x] * (Ksc[j] * expf(Lc[t] - Lc[j])) : 0.f;
       }
       *(float4*)(AT + (size_t)j * CP + t0 + 4 * lg) = o;
     }
@@ -314,21 +329,33 @@ __global__ __launch_bounds__(256) void state_chunks_kernel(ScanArgs a, int C, Sp
         if (lane == 0) Rs[t] = 1.0f / sqrtf(ss / (float)P + a.eps);
       }
     // (a wave reads the Rs it wrote itself: tokens wave, wave + 4, ...)
-    for (int pb = 0; outputs && pb < P; pb += 64) {
-      const int pc = min(pb + lane, P - 1);
-      for (int tb = wave; tb < m; tb += 32) {
-        float gv[8];
+    if (gates_ahead || (outputs && !a.gate && P <= 64)) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          gv[u] = a.gate ? a.gate[(row0 + min(tb + 4 * u, m - 1)) * a.ldg + (size_t)h * P + pc] : 0.f;
+      for (int u = 0; u < 16; ++u) {
+        const int t = wave + 4 * u;
+        if (t >= m || lane >= P) continue;
+        float o = O[(size_t)t * Pp + lane];
+        if (a.unit_rms) o *= Rs[t];
+        if (a.gate) o *= silu_f(gv[u]);
+        ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + lane] = from_f32<T>(o);
+      }
+    } else {
+      for (int pb = 0; outputs && pb < P; pb += 64) {
+        const int pc = min(pb + lane, P - 1);
+        for (int tb = wave; tb < m; tb += 32) {
+          float g8[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int t = tb + 4 * u;
-          if (t >= m || pb + lane >= P) continue;
-          float o = O[(size_t)t * Pp + pc];
-          if (a.unit_rms) o *= Rs[t];
-          if (a.gate) o *= silu_f(gv[u]);
-          ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + pc] = from_f32<T>(o);
+          for (int u = 0; u < 8; ++u)
+            g8[u] = a.gate ? a.gate[(row0 + min(tb + 4 * u, m - 1)) * a.ldg + (size_t)h * P + pc] : 0.f;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const int t = tb + 4 * u;
+            if (t >= m || pb + lane >= P) continue;
+            float o = O[(size_t)t * Pp + pc];
+            if (a.unit_rms) o *= Rs[t];
+            if (a.gate) o *= silu_f(g8[u]);
+            ((T*)a.out)[(row0 + t) * a.ldo + (size_t)h * P + pc] = from_f32<T>(o);
+          }
         }
       }
     }
