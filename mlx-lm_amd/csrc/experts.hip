@@ -100,54 +100,106 @@ __device__ __forceinline__ float lane_dot(const T* __restrict__ a, const T* __re
   return s;
 }
 
-// Block (token x pick, feature group): a wave a feature at a time, lanes along the width.
+// ROWS dot products of one vector b with ROWS rows a[r], all loads of a step on their way at once.
+template <typename T, bool VEC, int ROWS>
+__device__ __forceinline__ void lane_dots(const T* const* __restrict__ a, const T* __restrict__ b, int K, int lane, float* s) {
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) s[r] = 0.f;
+  if (VEC) {
+    constexpr int W = 16 / sizeof(T);
+    for (int k = lane * W; k < K; k += 64 * W) {
+      u32x4_t av[ROWS];
+      const u32x4_t bv = *(const u32x4_t*)(b + k);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) av[r] = *(const u32x4_t*)(a[r] + k);
+      const T* bp = (const T*)&bv;
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) {
+        const T* ap = (const T*)&av[r];
+#pragma unroll
+        for (int i = 0; i < W; ++i) s[r] += to_f32(ap[i]) * to_f32(bp[i]);
+      }
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) {
+      const float bv = to_f32(b[k]);
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) s[r] += to_f32(a[r][k]) * bv;
+    }
+  }
+}
+
+// Block (token x pick, 16 features): a wave four features at once (eight rows of weights in
+// flight), lanes along the width.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void expert_rows_up_kernel(const T* __restrict__ x, int ldx,
                                                              const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                              const int* __restrict__ idx,
                                                              const float* __restrict__ weight, int n_experts, int top,
-                                                             int F, int width, T* __restrict__ act, int feats_a_block) {
+                                                             int F, int width, T* __restrict__ act) {
   const int item = blockIdx.x, t = item / top;
   const int e = idx[item];
   if (e >= n_experts) return;  // an identity expert: nothing to compute
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int f0 = blockIdx.y * 16 + wave * 4;
+  if (f0 >= F) return;  // (no barrier in this kernel)
+  const T* rows[8];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const size_t f = (size_t)e * F + min(f0 + r, F - 1);
+    rows[r] = w_gate + f * width, rows[4 + r] = w_up + f * width;
+  }
+  float s[8];
+  lane_dots<T, VEC, 8>(rows, x + (size_t)t * ldx, width, lane, s);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) s[r] = wave_sum(s[r]);
   const float wt = weight[item];
-  const T* xr = x + (size_t)t * ldx;
-  const int f_end = min(F, ((int)blockIdx.y + 1) * feats_a_block);
-  for (int f = blockIdx.y * feats_a_block + wave; f < f_end; f += 4) {
-    const float sg = wave_sum(lane_dot<T, VEC>(w_gate + ((size_t)e * F + f) * width, xr, width, lane));
-    const float su = wave_sum(lane_dot<T, VEC>(w_up + ((size_t)e * F + f) * width, xr, width, lane));
-    if (lane == 0) act[(size_t)item * F + f] = from_f32<T>(wt * silu_f(sg) * su);
+  if (lane < 4 && f0 + lane < F) {
+    float g = s[0], u = s[4];
+#pragma unroll
+    for (int r = 1; r < 4; ++r)
+      if (lane == r) g = s[r], u = s[4 + r];
+    act[(size_t)item * F + f0 + lane] = from_f32<T>(wt * silu_f(g) * u);
   }
 }
 
-// Block (token, column group): a wave an output column at a time, lanes along the features.
+// Block (token, 16 columns): a wave four output columns at once, lanes along the features.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void expert_rows_down_kernel(const T* __restrict__ act, const T* __restrict__ w_down,
                                                                const int* __restrict__ idx,
                                                                const float* __restrict__ weight,
                                                                const T* __restrict__ x, int ldx, int n_experts, int top,
                                                                int F, int width, float* __restrict__ y, int ldy,
-                                                               int cols_a_block, int accumulate) {
+                                                               int accumulate) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n_end = min(width, ((int)blockIdx.y + 1) * cols_a_block);
-  for (int n = blockIdx.y * cols_a_block + wave; n < n_end; n += 4) {
-    float s = 0.f, same = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const int e = idx[(size_t)t * top + j];
-      if (e >= n_experts) {
-        same += weight[(size_t)t * top + j];
-        continue;
-      }
-      s += lane_dot<T, VEC>(w_down + ((size_t)e * width + n) * F, act + ((size_t)t * top + j) * F, F, lane);
+  const int n0 = blockIdx.y * 16 + wave * 4;
+  if (n0 >= width) return;
+  float tot[4] = {0.f, 0.f, 0.f, 0.f}, same = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int e = idx[(size_t)t * top + j];
+    if (e >= n_experts) {
+      same += weight[(size_t)t * top + j];
+      continue;
     }
-    s = wave_sum(s);
-    if (lane == 0) {
-      const float v = s + same * to_f32(x[(size_t)t * ldx + n]);
-      float* o = y + (size_t)t * ldy + n;
-      *o = accumulate ? *o + v : v;
-    }
+    const T* rows[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) rows[r] = w_down + ((size_t)e * width + min(n0 + r, width - 1)) * F;
+    float s[4];
+    lane_dots<T, VEC, 4>(rows, act + ((size_t)t * top + j) * F, F, lane, s);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) tot[r] += s[r];
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) tot[r] = wave_sum(tot[r]);
+  if (lane < 4 && n0 + lane < width) {
+    float v = tot[0];
+#pragma unroll
+    for (int r = 1; r < 4; ++r)
+      if (lane == r) v = tot[r];
+    v += same * to_f32(x[(size_t)t * ldx + n0 + lane]);
+    float* o = y + (size_t)t * ldy + n0 + lane;
+    *o = accumulate ? *o + v : v;
   }
 }
 
@@ -427,17 +479,16 @@ extern "C" int expert_rows(const void* x, int ldx, const void* w_gate, const voi
     FAIL("expert_rows: null pointer");
   if (top <= 0 || F <= 0 || width <= 0 || ldx < width || ldy < width) FAIL("expert_rows: sizes");
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("expert_rows: unknown dtype code %d", dtype);
-  // (few features and columns a block: a step of one token still puts a block on every CU)
-  const int feats = 8, cols = 8, per = dtype == DT_BF16 ? 8 : 4;
+  const int feats = 16, cols = 16, per = dtype == DT_BF16 ? 8 : 4;
   const bool vec = F % per == 0 && width % per == 0 && ldx % per == 0 && !((uintptr_t)x & 15);
   dim3 block(256), up_grid(n_tokens * top, (F + feats - 1) / feats), down_grid(n_tokens, (width + cols - 1) / cols);
 #define RUN(T, VEC)                                                                                                        \
   do {                                                                                                                     \
     if (n_experts > 0)                                                                                                     \
       hipLaunchKernelGGL((expert_rows_up_kernel<T, VEC>), up_grid, block, 0, stream, (const T*)x, ldx, (const T*)w_gate,   \
-                         (const T*)w_up, idx, weight, n_experts, top, F, width, (T*)act, feats);                           \
+                         (const T*)w_up, idx, weight, n_experts, top, F, width, (T*)act);                           \
     hipLaunchKernelGGL((expert_rows_down_kernel<T, VEC>), down_grid, block, 0, stream, (const T*)act, (const T*)w_down,    \
-                       idx, weight, (const T*)x, ldx, n_experts, top, F, width, y, ldy, cols, accumulate);                 \
+                       idx, weight, (const T*)x, ldx, n_experts, top, F, width, y, ldy, accumulate);                 \
   } while (0)
   if (dtype == DT_F32) {
     if (vec) RUN(float, true); else RUN(float, false);
