@@ -23,13 +23,8 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 // A wave a token, up to ROUTER_PER_LANE outputs a lane.  The k-th pick is the largest choice score
 // not picked yet, the lowest index on a tie.
 #define ROUTER_PER_LANE 8
-__global__ __launch_bounds__(256) void router_choice_kernel(const float* __restrict__ z, int ldz,
-                                                            const float* __restrict__ correction, int n_tokens,
-                                                            int n_out, int top, int* __restrict__ idx,
-                                                            float* __restrict__ weight) {
-  const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= n_tokens) return;  // whole waves leave; no barrier follows
-  const float* zr = z + (size_t)t * ldz;
+__device__ __forceinline__ void route_token(const float* __restrict__ zr, const float* __restrict__ correction, int n_out,
+                                            int top, int* __restrict__ idx, float* __restrict__ weight, int lane) {
   float v[ROUTER_PER_LANE], c[ROUTER_PER_LANE];
   float m = -INFINITY;
 #pragma unroll
@@ -65,10 +60,32 @@ __global__ __launch_bounds__(256) void router_choice_kernel(const float* __restr
 #pragma unroll
     for (int i = 0; i < ROUTER_PER_LANE; ++i)
       if (lane + 64 * i == e) {
-        idx[(size_t)t * top + j] = e, weight[(size_t)t * top + j] = v[i];
+        idx[j] = e, weight[j] = v[i];
         c[i] = -INFINITY;  // picked
       }
   }
+}
+
+__global__ __launch_bounds__(256) void router_choice_kernel(const float* __restrict__ z, int ldz,
+                                                            const float* __restrict__ correction, int n_tokens,
+                                                            int n_out, int top, int* __restrict__ idx,
+                                                            float* __restrict__ weight) {
+  const int lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= n_tokens) return;  // whole waves leave; no barrier follows
+  route_token(z + (size_t)t * ldz, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane);
+}
+
+// For a step of few tokens, where one product gave [router | gate | up] as float rows: a block a
+// token, its first wave chooses the experts, all of it makes act = silu(gate) * up.
+template <typename T>
+__global__ __launch_bounds__(256) void route_and_gate_kernel(const float* __restrict__ zu, int ld,
+                                                             const float* __restrict__ correction, int n_out, int top,
+                                                             int F, int* __restrict__ idx, float* __restrict__ weight,
+                                                             T* __restrict__ act, int ldo) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const float* row = zu + (size_t)t * ld;
+  if (threadIdx.x < 64) route_token(row, correction, n_out, top, idx + (size_t)t * top, weight + (size_t)t * top, lane);
+  for (int f = threadIdx.x; f < F; f += 256) act[(size_t)t * ldo + f] = from_f32<T>(silu_f(row[n_out + f]) * row[n_out + F + f]);
 }
 
 template <typename T>
@@ -453,6 +470,24 @@ extern "C" int router_choice(const float* z, int ldz, const float* correction, i
   hipLaunchKernelGGL(router_choice_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, ldz, correction,
                      n_tokens, n_out, top, idx, weight);
   CHECK_LAUNCH("router_choice");
+  return 0;
+}
+
+extern "C" int route_and_gate(const float* zu, int ld, const float* correction, int n_tokens, int n_out, int top, int F,
+                              int* idx, float* weight, void* act, int ldo, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (!zu || !idx || !weight || !act) FAIL("route_and_gate: null pointer");
+  if (n_out <= 0 || top <= 0 || top > n_out || F <= 0 || ld < n_out + 2 * F || ldo < F)
+    FAIL("route_and_gate: %d of %d outputs and 2 x %d columns in rows of %d", top, n_out, F, ld);
+  if (n_out > 64 * ROUTER_PER_LANE) FAIL("route_and_gate: %d outputs, at most %d", n_out, 64 * ROUTER_PER_LANE);
+  if (dtype != DT_F32 && dtype != DT_BF16) FAIL("route_and_gate: unknown dtype code %d", dtype);
+  if (dtype == DT_F32)
+    hipLaunchKernelGGL(route_and_gate_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, zu, ld, correction, n_out, top, F,
+                       idx, weight, (float*)act, ldo);
+  else
+    hipLaunchKernelGGL(route_and_gate_kernel<bf16>, dim3(n_tokens), dim3(256), 0, stream, zu, ld, correction, n_out, top, F,
+                       idx, weight, (bf16*)act, ldo);
+  CHECK_LAUNCH("route_and_gate");
   return 0;
 }
 

@@ -1041,6 +1041,24 @@ def router_choice(idx, weight, z, correction, top):
     build.check(lib, rc, "router_choice")
 
 
+def route_and_gate(idx, weight, act, zu, correction, top, n_out):
+    """``router_choice`` on the first ``n_out`` columns of the float32 rows ``zu`` and ``silu_mul`` on
+    the ``2 * act.shape[1]`` columns behind them, in one launch (for steps of few tokens)."""
+    lib = build.load("experts")
+    ld, ldo = _f32_rows(zu, "zu", 1), _rows2d(act, "act")
+    T, F = act.shape
+    _need(zu.shape[0] >= T and zu.shape[1] == n_out + 2 * F and act.dtype in DT, "route_and_gate: shapes")
+    _dev(idx, "idx", torch.int32)
+    _dev(weight, "weight", torch.float32)
+    _need(idx.numel() >= T * top and weight.numel() >= T * top, "route_and_gate: idx / weight too short")
+    if correction is not None:
+        _dev(correction, "correction", torch.float32)
+        _need(correction.numel() == n_out, "route_and_gate: correction length")
+    rc = lib.route_and_gate(_ptr(zu), _c_int(ld), _ptr(correction), _c_int(T), _c_int(n_out), _c_int(top), _c_int(F),
+                            _ptr(idx), _ptr(weight), _ptr(act), _c_int(ldo), _c_int(DT[act.dtype]), _stream())
+    build.check(lib, rc, "route_and_gate")
+
+
 def silu_mul(out, gate_up):
     """``out = silu(gate_up[:, :F]) * gate_up[:, F:2F]`` with ``F = out.shape[1]``."""
     lib = build.load("experts")

@@ -29,6 +29,7 @@ class GatedExperts(FeedForward):
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
     can_overwrite = True
+    MERGED_UP_TO = 16  # up to this many tokens the router's and the shared expert's first products are one
     TILES_FROM = 64  # from this many tokens in a step the picks are sorted and go to the matrix cores in tiles
 
     def __init__(self, width, n_experts, inner, top, n_identity=0, shared_inner=0, correction=True, prefix=""):
@@ -82,17 +83,28 @@ class GatedExperts(FeedForward):
                 d = torch.cat([d, d.new_zeros(self.width, pad)], 1)
             self.shared_in = kernels.for_decode(torch.cat([g, u]).contiguous())
             self.shared_out = kernels.for_decode(d.contiguous())
+            # for steps of few tokens: router, gate and up in one product (float32 rows)
+            self.merged_in = kernels.for_decode(torch.cat([tensors[n("router")], g, u]).contiguous())
 
     def forward(self, ctx, x, residual):
         T = x.shape[0]
         mark = ctx.scratch_mark()
-        z = ctx.scratch((T, self.n_out), torch.float32)
-        kernels.linear(z, x, self.router_w, splits=kernels.splits_alone(T))
         idx = ctx.scratch((T, self.top), torch.int32)
         weight = ctx.scratch((T, self.top), torch.float32)
-        kernels.router_choice(idx, weight, z, self.correction, self.top)
         accumulate = not self.overwrite
-        if self.shared_inner:
+        if self.shared_inner and T <= self.MERGED_UP_TO:
+            # few tokens: what a launch costs counts for more than what it computes
+            zu = ctx.scratch((T, self.n_out + 2 * self.shared_padded), torch.float32)
+            kernels.linear(zu, x, self.merged_in)
+            act = ctx.scratch((T, self.shared_padded), ctx.dtype)
+            kernels.route_and_gate(idx, weight, act, zu, self.correction, self.top, self.n_out)
+            kernels.linear(residual, act, self.shared_out, accumulate=accumulate)
+            accumulate = True
+        else:
+            z = ctx.scratch((T, self.n_out), torch.float32)
+            kernels.linear(z, x, self.router_w, splits=kernels.splits_alone(T))
+            kernels.router_choice(idx, weight, z, self.correction, self.top)
+        if self.shared_inner and T > self.MERGED_UP_TO:
             gu = ctx.scratch((T, 2 * self.shared_padded), ctx.dtype)
             kernels.linear(gu, x, self.shared_in, splits=kernels.splits_alone(T))
             act = ctx.scratch((T, self.shared_padded), ctx.dtype)

@@ -337,6 +337,26 @@ def test_the_routers_choice(n_out, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_choice_and_gate_in_one_launch(dtype):
+    """For steps of few tokens one product gives [router | gate | up] and one kernel chooses the
+    experts and makes silu(gate) * up."""
+    from mlx_lm_amd.ops import kernels
+
+    g = torch.Generator().manual_seed(7)
+    T, n_out, top, F = 5, 11, 3, 40
+    zu = torch.randn(T, n_out + 2 * F, generator=g) * 2
+    corr = torch.randn(n_out, generator=g) * 0.1
+    idx, w = torch.empty(T, top, dtype=torch.int32, device="cuda"), torch.empty(T, top, device="cuda")
+    act = torch.empty(T, F, dtype=dtype, device="cuda")
+    kernels.route_and_gate(idx, w, act, zu.cuda(), corr.cuda(), top, n_out)
+    s = torch.softmax(zu[:, :n_out].double(), -1)
+    want = torch.topk(s + corr.double(), top, -1).indices
+    assert torch.equal(idx.cpu().long(), want) and (w.double().cpu() - torch.gather(s, 1, want)).abs().max() <= 1e-6
+    gated = plain.silu(zu[:, n_out : n_out + F].double()) * zu[:, n_out + F :].double()
+    assert (act.double().cpu() - gated).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2) * gated.abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,width,F", [(1, 64, 24), (9, 72, 10), (40, 256, 64), (300, 72, 40), (70, 104, 8)])
 def test_chosen_experts_and_identity_experts(dtype, T, width, F):
     from mlx_lm_amd.ops import kernels
