@@ -418,9 +418,9 @@ __global__ __launch_bounds__(256) void rotate_pairs_kernel(float* __restrict__ q
 __global__ __launch_bounds__(256) void ssm_prepare_kernel(
     const float* __restrict__ u, int ldu, int conv_col, int dt_col, const float* __restrict__ w,
     const float* __restrict__ b, int taps, int C, int H, const float* __restrict__ dt_bias,
-    const float* __restrict__ A_log, const float* __restrict__ state, size_t state_stride, size_t conv_offset,
+    const float* __restrict__ A_log, float* __restrict__ state, size_t state_stride, size_t conv_offset,
     const int* __restrict__ token_req, const int* __restrict__ seq_start, const int* __restrict__ slot_ids,
-    float* __restrict__ xbc, float* __restrict__ dt, float* __restrict__ log_a, int n_tokens) {
+    float* __restrict__ xbc, float* __restrict__ dt, float* __restrict__ log_a, int n_tokens, int single_tokens) {
   const int c = blockIdx.y * 256 + threadIdx.x, row = blockIdx.x;
   if (c >= C + H) return;
   if (c >= C) {
@@ -431,12 +431,15 @@ __global__ __launch_bounds__(256) void ssm_prepare_kernel(
     return;
   }
   const int req = token_req[row], local = row - seq_start[req];
-  const float* old = state + (size_t)slot_ids[req] * state_stride + conv_offset;  // [taps - 1, C], the latest last
+  float* old = state + (size_t)slot_ids[req] * state_stride + conv_offset;  // [taps - 1, C], the latest last
   float acc = b ? b[c] : 0.f;
   for (int j = taps - 1; j >= 0; --j) {  // the oldest input first
     const int at = local - j;
     const float in = at >= 0 ? u[(size_t)(row - j) * ldu + conv_col + c] : old[(size_t)(taps - 1 + at) * C + c];
     acc += w[(size_t)c * taps + (taps - 1 - j)] * in;
+    // every request brings one token: this thread is the only one that reads or writes its
+    // request's inputs of channel c, so it moves them up by one as it goes (the oldest first)
+    if (single_tokens && j < taps - 1) old[(size_t)(taps - 2 - j) * C + c] = in;
   }
   xbc[(size_t)row * C + c] = silu_f(acc);
 }
@@ -573,10 +576,13 @@ extern "C" int state_scan(const ScanArgs* args, int chunked, int span, int n_spa
   return 0;
 }
 
+// `single_tokens`: every request brings one token (the caller says so); the kernel then also moves
+// the requests' last inputs up by one, and no conv_state_update follows.
 extern "C" int ssm_prepare(const float* u, int ldu, int conv_col, int dt_col, const float* w, const float* b, int taps,
-                           int C, int H, const float* dt_bias, const float* A_log, const float* state,
+                           int C, int H, const float* dt_bias, const float* A_log, float* state,
                            size_t state_stride, size_t conv_offset, const int* token_req, const int* seq_start,
-                           const int* slot_ids, float* xbc, float* dt, float* log_a, int n_tokens, hipStream_t stream) {
+                           const int* slot_ids, float* xbc, float* dt, float* log_a, int n_tokens, int single_tokens,
+                           hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (!u || !w || !dt_bias || !A_log || !state || !token_req || !seq_start || !slot_ids || !xbc || !dt || !log_a)
     FAIL("ssm_prepare: null pointer");
@@ -584,7 +590,7 @@ extern "C" int ssm_prepare(const float* u, int ldu, int conv_col, int dt_col, co
     FAIL("ssm_prepare: %d taps, %d channels from column %d, %d heads from column %d, rows of %d", taps, C, conv_col, H, dt_col, ldu);
   dim3 grid(n_tokens, (C + H + 255) / 256), block(256);
   hipLaunchKernelGGL(ssm_prepare_kernel, grid, block, 0, stream, u, ldu, conv_col, dt_col, w, b, taps, C, H, dt_bias,
-                     A_log, state, state_stride, conv_offset, token_req, seq_start, slot_ids, xbc, dt, log_a, n_tokens);
+                     A_log, state, state_stride, conv_offset, token_req, seq_start, slot_ids, xbc, dt, log_a, n_tokens, single_tokens);
   CHECK_LAUNCH("ssm_prepare");
   return 0;
 }

@@ -964,10 +964,11 @@ def state_scan(out, q, k, v, state, state_offset, seq_start, seq_len, slot_ids, 
 
 
 def ssm_prepare(xbc, dt, log_a, u, conv_col, dt_col, conv_w, conv_b, dt_bias, a_log, state, conv_offset, token_req,
-                seq_start, slot_ids):
+                seq_start, slot_ids, single_tokens=False):
     """The causal convolution (with the requests' last inputs from ``state``), bias and silu of
     columns ``conv_col ..`` of the float32 rows ``u`` into ``xbc``; ``dt = softplus(u[:, dt_col + h]
-    + dt_bias[h])`` and ``log_a = -exp(a_log[h]) * dt`` (csrc/linear_state.hip)."""
+    + dt_bias[h])`` and ``log_a = -exp(a_log[h]) * dt`` (csrc/linear_state.hip).  ``single_tokens``:
+    every request brings one token, and the kernel also does what ``conv_state_update`` would."""
     lib = build.load("linear_state")
     ldu = _f32_rows(u, "u", 1)
     T, C = xbc.shape
@@ -988,7 +989,8 @@ def ssm_prepare(xbc, dt, log_a, u, conv_col, dt_col, conv_w, conv_b, dt_bias, a_
     rc = lib.ssm_prepare(_ptr(u), _c_int(ldu), _c_int(conv_col), _c_int(dt_col), _ptr(conv_w), _ptr(conv_b),
                          _c_int(taps), _c_int(C), _c_int(H), _ptr(dt_bias), _ptr(a_log), _ptr(state),
                          _c_size_t(state.stride(0)), _c_size_t(conv_offset), _ptr(token_req), _ptr(seq_start),
-                         _ptr(slot_ids), _ptr(xbc), _ptr(dt), _ptr(log_a), _c_int(T), _stream())
+                         _ptr(slot_ids), _ptr(xbc), _ptr(dt), _ptr(log_a), _c_int(T), _c_int(int(bool(single_tokens))),
+                         _stream())
     build.check(lib, rc, "ssm_prepare")
 
 

@@ -209,10 +209,13 @@ class StateSpace(_SequenceArrays, Mixer):
         dt = ctx.scratch((T, H), torch.float32)
         log_a = ctx.scratch((T, H), torch.float32)
         starts, lens = ctx.array("sequences.starts"), ctx.array("sequences.lens")
+        single = ctx.array("sequences.longest") == 1  # a decode step: the convolution's kernel keeps the state itself
         kernels.ssm_prepare(xbc, dt, log_a, u, self.inner, self.inner + self.channels, self.conv_w, self.conv_b,
-                            self.dt_bias, self.a_log, cache.state, 0, ctx.token_req, starts, ctx.slot_ids)
-        kernels.conv_state_update(u, self.inner, self.taps, self.channels, cache.state, 0, starts, lens, ctx.slot_ids,
-                                  ctx.n_requests)
+                            self.dt_bias, self.a_log, cache.state, 0, ctx.token_req, starts, ctx.slot_ids,
+                            single_tokens=single)
+        if not single:
+            kernels.conv_state_update(u, self.inner, self.taps, self.channels, cache.state, 0, starts, lens, ctx.slot_ids,
+                                      ctx.n_requests)
         y = ctx.scratch((T, self.inner), torch.float32)
         kernels.state_scan(y, xbc[:, self.inner + GN:], xbc[:, self.inner:self.inner + GN], xbc[:, :self.inner],
                            cache.state, self.conv_floats, starts, lens, ctx.slot_ids, ctx.n_requests, H, self.groups,

@@ -287,8 +287,9 @@ def test_the_convolution_across_portions(taps):
         xbc, dt, la = torch.empty(2 * m, C, device="cuda"), torch.empty(2 * m, H, device="cuda"), torch.empty(2 * m, H, device="cuda")
         req = _ints([0] * m + [1] * m)
         kernels.ssm_prepare(xbc, dt, la, rows, pad, pad + C, w.cuda(), b.cuda(), dt_bias.cuda(), a_log.cuda(), state, 4, req,
-                            _ints([0, m]), _ints([2, 1]))
-        kernels.conv_state_update(rows, pad, taps, C, state, 4, _ints([0, m]), _ints([m, m]), _ints([2, 1]), 2)
+                            _ints([0, m]), _ints([2, 1]), single_tokens=m == 1)  # (one token each: the kernel keeps the state itself)
+        if m > 1:
+            kernels.conv_state_update(rows, pad, taps, C, state, 4, _ints([0, m]), _ints([m, m]), _ints([2, 1]), 2)
         got[0].append(xbc[:m].cpu()), got[1].append(xbc[m:].cpu())
         got_dt.append(dt[:m].cpu()), got_a.append(la[:m].cpu())
         at += m
