@@ -2,9 +2,11 @@
 //   router_choice   s = softmax(z) over all router outputs; the `top` largest of s + correction
 //                   are chosen (the lower index on a tie); their weights are s itself.
 //   silu_mul        act = silu(gate) * up for rows [gate | up]   (a dense gated feed-forward)
+//   route_and_gate  both of these in one launch, for a step of few tokens whose router, gate and up
+//                   came out of one product as float rows
 //   expert_rows_up / expert_rows_down
 //                   a token's chosen experts read straight from the stacked expert weights, a
-//                   wave a feature: act[t, j, :] = w_tj silu(Wg_e x_t) * (Wu_e x_t), then
+//                   wave four features at once: act[t, j, :] = w_tj silu(Wg_e x_t) * (Wu_e x_t), then
 //                   y[t, :] += sum_j Wd_e act[t, j, :] + sum_(j: e is an identity expert) w_tj x_t.
 //                   Only the chosen experts' weights are read: the kernels for few tokens.
 //   expert_tiles    the same for many tokens: the picks are sorted by expert on the device
@@ -97,27 +99,8 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gu,
   out[(size_t)r * ldo + f] = from_f32<T>(silu_f(to_f32(row[f])) * to_f32(row[F + f]));
 }
 
-// sum_k a[k] b[k] over a lane's share of K: 16 bytes a lane and load where K and both rows allow
-// (VEC), a value a lane otherwise.
-template <typename T, bool VEC>
-__device__ __forceinline__ float lane_dot(const T* __restrict__ a, const T* __restrict__ b, int K, int lane) {
-  float s = 0.f;
-  if (VEC) {
-    constexpr int W = 16 / sizeof(T);
-    for (int k = lane * W; k < K; k += 64 * W) {
-      const u32x4_t av = *(const u32x4_t*)(a + k), bv = *(const u32x4_t*)(b + k);
-      const T* ap = (const T*)&av;
-      const T* bp = (const T*)&bv;
-#pragma unroll
-      for (int i = 0; i < W; ++i) s += to_f32(ap[i]) * to_f32(bp[i]);
-    }
-  } else {
-    for (int k = lane; k < K; k += 64) s += to_f32(a[k]) * to_f32(b[k]);
-  }
-  return s;
-}
-
-// ROWS dot products of one vector b with ROWS rows a[r], all loads of a step on their way at once.
+// ROWS dot products of one vector b with ROWS rows a[r] over a lane's share of K, all loads of a step on
+// their way at once: 16 bytes a lane and load where K and the rows allow (VEC), a value a lane otherwise.
 template <typename T, bool VEC, int ROWS>
 __device__ __forceinline__ void lane_dots(const T* const* __restrict__ a, const T* __restrict__ b, int K, int lane, float* s) {
 #pragma unroll
